@@ -14,3 +14,7 @@ from . import pupalorn as _pupalorn
 from .pupalorn import PupalornConfig
 
 register_architecture(_pupalorn.ARCHITECTURE, PupalornConfig.from_dict, _pupalorn.build_plan)
+from . import kosalorn as _kosalorn
+from .kosalorn import KosalornConfig
+
+register_architecture(_kosalorn.ARCHITECTURE, KosalornConfig.from_dict, _kosalorn.build_plan)

@@ -69,10 +69,13 @@ class LayerCall:
     `layer` indexes `ModelPlan.layers`. `cache_of` names the entry of the run
     order whose cache this call reads instead of owning one (None: its own).
     A layer may be called more than once; each call that owns a cache gets its
-    own cache site.
+    own cache site. `add_input`: the embedding's output (the stream as it was
+    before the first layer) is added to the stream before this call runs, as a
+    looped model does at the start of every pass after the first.
     """
     layer: int
     cache_of: Optional[int] = None
+    add_input: bool = False
 
 
 @dataclass(frozen=True)

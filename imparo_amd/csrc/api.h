@@ -115,6 +115,48 @@ int imparo_attention_dv(const void* q, const void* k_cache, const void* v_cache,
                         int n_tokens, int heads, int kv_heads, int head_dim, int value_dim, int out_ld, int n_pages,
                         float scale, int window, int v_transposed, imparo_stream stream);
 
+// ---- attention over a cached latent (absorbed form)
+// Attention in which every head reads the same cached rows [pages, page, row_dim]: a key is a whole row, its value
+// the row's first value_dim numbers. q [tokens, heads, row_dim], out [tokens, heads * value_dim].
+int imparo_attention_latent(const void* q, const void* rows_cache, void* out, int dtype, const int32_t* positions,
+                            const int32_t* row_of_token, const int32_t* block_table, int table_stride, int page_size,
+                            int n_tokens, int heads, int row_dim, int value_dim, int n_pages, float scale, int window,
+                            imparo_stream stream);
+// Per token: the first `rank` numbers of kv_rows [tokens, rank + rot_dim] are divided by their root mean square
+// (eps inside the root) and multiplied by norm_weight; the last rot_dim are turned by position (the first
+// 2 n_freq of them; pair i is (i, i + n_freq), or with `interleaved` (2i, 2i + 1); angle = position *
+// inv_freq[i]); the row goes to the token's place in `cache` [pages, page, rank + rot_dim] (cache null: not
+// written). q_rows [tokens, heads * (dim + rot_dim)]: each head's first dim numbers go to q_plain [tokens, heads,
+// dim], its last rot_dim, turned alike, to columns rank .. of q_full [tokens, heads, rank + rot_dim].
+int imparo_latent_store(const float* q_rows, const float* kv_rows, const float* norm_weight, float eps,
+                        const float* inv_freq, int n_freq, int interleaved, const int32_t* positions,
+                        const int32_t* row_of_token, const int32_t* block_table, int table_stride, int page_size,
+                        int n_pages, void* cache, void* q_plain, void* q_full, int dtype, int n_tokens, int heads,
+                        int dim, int rot_dim, int rank, imparo_stream stream);
+// out[t, h, :n] = W[h] in[t, h, :k] with w [heads, k, n]: a token's rows lie in_ld (out_ld) apart, a head's part
+// in_hs (out_hs) apart inside a row. float32 sums in the order of k.
+int imparo_head_gemm(const void* in, int in_ld, int in_hs, const void* w, int dtype, void* out, int out_dtype,
+                     int out_ld, int out_hs, int n_tokens, int heads, int k, int n, imparo_stream stream);
+
+// ---- a gated linear recurrence with a matrix of state a head
+// Per request (row), head and token in order: q = silu(zq), f = lower + (1 - lower) sigmoid(zf),
+// S <- diag(f) S + (1 - f) v^T, out = S^T q. rows [tokens, ld] float32 holds zq at q_off, zf at f_off, v at v_off,
+// head by head; state [slots, heads, dim, vdim] float32; out [tokens, heads * vdim] float32. dim <= 256.
+int imparo_hgrn2_scan(const float* rows, int ld, int q_off, int f_off, int v_off, const float* lower, float* state,
+                      const int32_t* seg_start, const int32_t* seg_len, const int32_t* slot, float* out, int n_rows,
+                      int heads, int dim, int vdim, imparo_stream stream);
+
+// ---- pieces of a parallel block with gated sublayers
+// x += a * sigmoid(gates[:, :width]) (+ b * sigmoid(gates[:, width : 2 width]), b may be null); with `copy`
+// the new x is also stored there in copy_dtype. x, a, b float32 [tokens, width]; gates float32 [tokens, gate_ld].
+int imparo_gated_sum(float* x, const float* a, const float* b, const float* gates, int gate_ld, void* copy,
+                     int copy_dtype, int n_tokens, int width, imparo_stream stream);
+// out[t, j] = gelu_tanh(z[t, j]) * table[ids[t], offset + j] for j < dim, zero for dim <= j < out_ld.
+int imparo_side_gate(const float* z, const void* table, int table_dtype, int table_ld, int offset, const int32_t* ids,
+                     int vocab, void* out, int out_dtype, int n_tokens, int dim, int out_ld, imparo_stream stream);
+// x[i] += y[i] for i < n.
+int imparo_add_rows(float* x, const float* y, long long n, imparo_stream stream);
+
 // Matrix-core attention, bfloat16, V cache transposed, page_size a power of two
 // >= 16, head_dim a multiple of 16 up to 128.
 // Decode: one query token per listed row (rows[i] indexes seg_start); the key
@@ -428,10 +470,16 @@ int imparo_embed_gather_scaled(const void* table, int table_dtype, const int32_t
                                int n_tokens, int width, int vocab, float scale, imparo_stream stream);
 
 // ---- a routed feed-forward (mixture of experts)
-// route: scores = softmax(logits[t, :n_router]); the `top` largest of score + correction are chosen (of equal
-// ones the lowest index), choice [tokens, top] holds their indices and weight [tokens, top] their scores.
+// route: scores = softmax(logits[t, :n_router]) (scoring 0) or the sigmoid of each output (scoring 1); the `top`
+// largest of score + correction are chosen (of equal ones the lowest index), choice [tokens, top] holds their
+// indices and weight [tokens, top] their scores.
 int imparo_moe_route(const float* logits, const float* correction, int32_t* choice, float* weight,
-                     int n_tokens, int n_router, int top, imparo_stream stream);
+                     int n_tokens, int n_router, int top, int scoring, imparo_stream stream);
+// hidden[slot, j] = silu(w g) * (w u), g = gu[slot, j], u = gu[slot, half + j], w = weight[entry_of_slot[slot]]
+// (weight null: 1): the hidden values of gated experts without biases that read w times their input, from the
+// stacked gate and up products of the input itself. gu float32 [n_slots, 2 half].
+int imparo_moe_gated(const float* gu, const float* weight, const int32_t* entry_of_slot, void* hidden, int out_dtype,
+                     int n_slots, int half, imparo_stream stream);
 // plan: entries are (token, choice) pairs in row-major order; those whose expert is below n_experts get a slot,
 // an expert's slots side by side (slot_of_entry, -1 for the others; entry_of_slot), and `tiles` [max_tiles, 3]
 // lists (expert, first slot, rows <= tile_rows) of every tile of rows, expert -1 past the list's end.
@@ -446,7 +494,8 @@ int imparo_moe_plan(const int32_t* choice, int n_entries, int n_experts, int til
 int imparo_moe_gemm(const void* a, int a_ld, int gather_div, const int32_t* entry_of_slot, const void* w,
                     void* out, int out_dtype, int dtype, const int32_t* tiles, int max_tiles, int tile_rows,
                     int n, int k, int epilogue, imparo_stream stream);
-// combine: out[t] = sum_j weight[t, j] * (y[slot of (t, j)] if choice[t, j] < n_experts else h[t]), j in order.
+// combine: out[t] = sum_j weight[t, j] * (y[slot of (t, j)] if choice[t, j] < n_experts else h[t]), j in order
+// (weight null: every weight is 1).
 int imparo_moe_combine(const float* y, const void* h, int h_dtype, const int32_t* choice,
                        const float* weight, const int32_t* slot_of_entry, float* out, int n_tokens,
                        int width, int top, int n_experts, imparo_stream stream);
@@ -454,7 +503,7 @@ int imparo_moe_combine(const float* y, const void* h, int h_dtype, const int32_t
 // route and plan in one launch, for at most imparo_moe_route_plan_tokens() tokens (a decode step)
 int imparo_moe_route_plan_tokens(void);
 int imparo_moe_route_plan(const float* logits, const float* correction, int32_t* choice, float* weight,
-                          int n_tokens, int n_router, int top, int n_experts, int tile_rows,
+                          int n_tokens, int n_router, int top, int scoring, int n_experts, int tile_rows,
                           int32_t* slot_of_entry, int32_t* entry_of_slot, int32_t* tiles, int max_tiles,
                           imparo_stream stream);
 

@@ -8,7 +8,7 @@
 #include "common.h"
 #include "api.h"
 
-#define ATT_MAX_HEAD_DIM 512
+#define ATT_MAX_HEAD_DIM 576
 #define ATT_WAVES 4
 
 template <typename T> struct Vec16;
@@ -59,7 +59,8 @@ __global__ void k_attention_wave(const T* __restrict__ q, const T* __restrict__ 
                                  T* __restrict__ out, const int32_t* __restrict__ positions,
                                  const int32_t* __restrict__ row_of_token, const int32_t* __restrict__ block_table,
                                  int table_stride, int page_size, int n_tokens, int heads, int kv_heads, int head_dim,
-                                 int value_dim, int out_ld, int n_pages, float scale, int window, int v_transposed) {
+                                 int value_dim, int out_ld, int n_pages, float scale, int window, int v_transposed,
+                                 int v_ld) {
     __shared__ float q_rows[ATT_WAVES][ATT_MAX_HEAD_DIM];
     __shared__ float probs[ATT_WAVES][WAVE];
     __shared__ long long v_off[ATT_WAVES][WAVE];
@@ -98,7 +99,7 @@ __global__ void k_attention_wave(const T* __restrict__ q, const T* __restrict__ 
                                                  : dot_row_any<T>(qr, k_cache + off, head_dim)) * scale;
                 // from here on `off` is where the key's value row starts
                 off = v_transposed ? ((long long)page * kv_heads + kvh) * page_size * value_dim + (p % page_size)
-                                   : (((long long)page * kv_heads + kvh) * page_size + (p % page_size)) * value_dim;
+                                   : (((long long)page * kv_heads + kvh) * page_size + (p % page_size)) * v_ld;
             }
         }
         const float m_new = fmaxf(m, wave_max(s));
@@ -151,15 +152,16 @@ static int check_attention_args(const void* q, const void* k_cache, const void* 
 // Keys of head_dim and values of value_dim a head: q [tokens, heads, head_dim], the value cache
 // [pages, kv_heads, page, value_dim] (or transposed inside the page), out [tokens, out_ld] with out_ld >=
 // heads * value_dim; what lies beyond the heads in a row is written as zeros.
-extern "C" int imparo_attention_dv(const void* q, const void* k_cache, const void* v_cache, void* out, int dtype,
-                                const int32_t* positions, const int32_t* row_of_token,
-                                const int32_t* block_table, int table_stride, int page_size,
-                                int n_tokens, int heads, int kv_heads, int head_dim, int value_dim, int out_ld,
-                                int n_pages, float scale, int window, int v_transposed, imparo_stream stream) {
+static int attention_wave(const void* q, const void* k_cache, const void* v_cache, void* out, int dtype,
+                          const int32_t* positions, const int32_t* row_of_token,
+                          const int32_t* block_table, int table_stride, int page_size,
+                          int n_tokens, int heads, int kv_heads, int head_dim, int value_dim, int out_ld,
+                          int n_pages, float scale, int window, int v_transposed, int v_ld, imparo_stream stream) {
     const int bad = check_attention_args(q, k_cache, v_cache, out, positions, row_of_token, block_table, table_stride,
                                          page_size, n_tokens, heads, kv_heads, head_dim, n_pages, window);
     if (bad) return bad;
     if (value_dim <= 0 || value_dim > ATT_MAX_HEAD_DIM || out_ld < heads * value_dim) return IMPARO_BAD_ARGUMENT;
+    if (v_ld < value_dim || (v_transposed && v_ld != value_dim)) return IMPARO_BAD_ARGUMENT;
     if (n_tokens == 0) return IMPARO_OK;
     const long long total = (long long)n_tokens * heads;
     const unsigned blocks = (unsigned)((total + ATT_WAVES - 1) / ATT_WAVES);
@@ -167,15 +169,40 @@ extern "C" int imparo_attention_dv(const void* q, const void* k_cache, const voi
     if (dtype == IMPARO_F32)
         k_attention_wave<float><<<blocks, ATT_WAVES * WAVE, 0, s>>>(
             (const float*)q, (const float*)k_cache, (const float*)v_cache, (float*)out, positions, row_of_token,
-            block_table, table_stride, page_size, n_tokens, heads, kv_heads, head_dim, value_dim, out_ld, n_pages, scale, window, v_transposed);
+            block_table, table_stride, page_size, n_tokens, heads, kv_heads, head_dim, value_dim, out_ld, n_pages, scale, window, v_transposed,
+            v_ld);
     else if (dtype == IMPARO_BF16)
         k_attention_wave<bf16_t><<<blocks, ATT_WAVES * WAVE, 0, s>>>(
             (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, (bf16_t*)out, positions, row_of_token,
             block_table, table_stride, page_size, n_tokens, heads, kv_heads, head_dim, value_dim, out_ld, n_pages, scale, window,
-            v_transposed);
+            v_transposed, v_ld);
     else
         return IMPARO_BAD_ARGUMENT;
     return launch_status();
+}
+
+extern "C" int imparo_attention_dv(const void* q, const void* k_cache, const void* v_cache, void* out, int dtype,
+                                const int32_t* positions, const int32_t* row_of_token,
+                                const int32_t* block_table, int table_stride, int page_size,
+                                int n_tokens, int heads, int kv_heads, int head_dim, int value_dim, int out_ld,
+                                int n_pages, float scale, int window, int v_transposed, imparo_stream stream) {
+    return attention_wave(q, k_cache, v_cache, out, dtype, positions, row_of_token, block_table, table_stride, page_size,
+                          n_tokens, heads, kv_heads, head_dim, value_dim, out_ld, n_pages, scale, window, v_transposed,
+                          value_dim, stream);
+}
+
+// Attention over a cached latent: every head reads the same rows [pages, page, row_dim]; a key is a whole
+// row, its value the row's first value_dim numbers (queries carry their side of the keys' up-projection,
+// the values' up-projection follows the weighted sum). out [tokens, heads * value_dim].
+extern "C" int imparo_attention_latent(const void* q, const void* rows_cache, void* out, int dtype,
+                                       const int32_t* positions, const int32_t* row_of_token,
+                                       const int32_t* block_table, int table_stride, int page_size, int n_tokens,
+                                       int heads, int row_dim, int value_dim, int n_pages, float scale, int window,
+                                       imparo_stream stream) {
+    if (value_dim > row_dim) return IMPARO_BAD_ARGUMENT;
+    return attention_wave(q, rows_cache, rows_cache, out, dtype, positions, row_of_token, block_table, table_stride,
+                          page_size, n_tokens, heads, 1, row_dim, value_dim, heads * value_dim, n_pages, scale, window, 0,
+                          row_dim, stream);
 }
 
 extern "C" int imparo_attention(const void* q, const void* k_cache, const void* v_cache, void* out, int dtype,

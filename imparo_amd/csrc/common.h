@@ -119,7 +119,10 @@ int imparo_load_code_attention_mfma();
 int imparo_load_code_decode_rows();
 int imparo_load_code_diff_attention();
 int imparo_load_code_elementwise();
+int imparo_load_code_gated_ops();
 int imparo_load_code_gemm();
+int imparo_load_code_hgrn2();
+int imparo_load_code_latent_attention();
 int imparo_load_code_moe();
 int imparo_load_code_rope_cache();
 int imparo_load_code_row_ops();

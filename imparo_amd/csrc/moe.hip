@@ -20,13 +20,15 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 #define MOE_MAX_ROUTER 512          // router outputs (experts of both kinds)
 #define MOE_MAX_EXPERTS 1024        // real experts the plan kernel keeps counters for
 #define MOE_MAX_TOP 16
+#define MOE_SCORE_SOFTMAX 0         // scores = softmax over all router outputs
+#define MOE_SCORE_SIGMOID 1         // scores = sigmoid of each output
 
 extern "C" int imparo_moe_max_tiles(int n_entries, int n_experts, int tile_rows);
 
 // ---------------------------------------------------------------- route
 __device__ __forceinline__ void moe_route_token(const float* __restrict__ logits, const float* __restrict__ correction,
                                                 int32_t* __restrict__ choice, float* __restrict__ weight, int t,
-                                                int n_router, int top) {
+                                                int n_router, int top, int scoring) {
     const int lane = threadIdx.x & (WAVE - 1);
     constexpr int PER = MOE_MAX_ROUTER / WAVE;
     float z[PER], pick[PER];
@@ -37,19 +39,26 @@ __device__ __forceinline__ void moe_route_token(const float* __restrict__ logits
         z[j] = i < n_router ? logits[(size_t)t * n_router + i] : -INFINITY;
         m = fmaxf(m, z[j]);
     }
-    m = wave_max(m);
-    float sum = 0.f;
+    if (scoring == MOE_SCORE_SIGMOID) {
+        // every output scored by itself
 #pragma unroll
-    for (int j = 0; j < PER; ++j) {
-        z[j] = (lane + j * WAVE) < n_router ? expf(z[j] - m) : 0.f;
-        sum += z[j];
+        for (int j = 0; j < PER; ++j) z[j] = (lane + j * WAVE) < n_router ? 1.0f / (1.0f + expf(-z[j])) : 0.f;
+    } else {
+        m = wave_max(m);
+        float sum = 0.f;
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            z[j] = (lane + j * WAVE) < n_router ? expf(z[j] - m) : 0.f;
+            sum += z[j];
+        }
+        sum = wave_sum(sum);
+        const float inv = 1.0f / sum;
+#pragma unroll
+        for (int j = 0; j < PER; ++j) z[j] *= inv;
     }
-    sum = wave_sum(sum);
-    const float inv = 1.0f / sum;
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
         const int i = lane + j * WAVE;
-        z[j] *= inv;
         pick[j] = i < n_router ? z[j] + (correction ? correction[i] : 0.f) : -INFINITY;
     }
     for (int k = 0; k < top; ++k) {
@@ -81,19 +90,20 @@ __device__ __forceinline__ void moe_route_token(const float* __restrict__ logits
 
 __global__ void k_moe_route(const float* __restrict__ logits, const float* __restrict__ correction,
                             int32_t* __restrict__ choice, float* __restrict__ weight, int n_tokens, int n_router,
-                            int top) {
+                            int top, int scoring) {
     const int t = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
-    if (t < n_tokens) moe_route_token(logits, correction, choice, weight, t, n_router, top);
+    if (t < n_tokens) moe_route_token(logits, correction, choice, weight, t, n_router, top, scoring);
 }
 
 extern "C" int imparo_moe_route(const float* logits, const float* correction, int32_t* choice, float* weight,
-                                int n_tokens, int n_router, int top, imparo_stream stream) {
+                                int n_tokens, int n_router, int top, int scoring, imparo_stream stream) {
     if (!logits || !choice || !weight || n_tokens < 0) return IMPARO_BAD_ARGUMENT;
+    if (scoring != MOE_SCORE_SOFTMAX && scoring != MOE_SCORE_SIGMOID) return IMPARO_BAD_ARGUMENT;
     if (n_router < 1 || n_router > MOE_MAX_ROUTER || top < 1 || top > n_router || top > MOE_MAX_TOP)
         return IMPARO_BAD_ARGUMENT;
     if (n_tokens == 0) return IMPARO_OK;
     k_moe_route<<<(n_tokens + 3) / 4, 4 * WAVE, 0, (hipStream_t)stream>>>(logits, correction, choice, weight, n_tokens,
-                                                                         n_router, top);
+                                                                         n_router, top, scoring);
     return launch_status();
 }
 
@@ -171,13 +181,14 @@ __global__ __launch_bounds__(1024) void k_moe_plan(const int32_t* __restrict__ c
 __global__ __launch_bounds__(1024) void k_moe_route_plan(const float* __restrict__ logits,
                                                          const float* __restrict__ correction,
                                                          int32_t* __restrict__ choice, float* __restrict__ weight,
-                                                         int n_tokens, int n_router, int top, int n_experts,
-                                                         int tile_rows, int32_t* __restrict__ slot_of_entry,
+                                                         int n_tokens, int n_router, int top, int scoring,
+                                                         int n_experts, int tile_rows,
+                                                         int32_t* __restrict__ slot_of_entry,
                                                          int32_t* __restrict__ entry_of_slot,
                                                          int32_t* __restrict__ tiles, int max_tiles) {
     __shared__ MoePlanShared sh;
     for (int t = threadIdx.x / WAVE; t < n_tokens; t += blockDim.x / WAVE)
-        moe_route_token(logits, correction, choice, weight, t, n_router, top);
+        moe_route_token(logits, correction, choice, weight, t, n_router, top, scoring);
     __threadfence_block();
     __syncthreads();
     moe_plan_block(sh, choice, n_tokens * top, n_experts, tile_rows, slot_of_entry, entry_of_slot, tiles, max_tiles);
@@ -186,10 +197,11 @@ __global__ __launch_bounds__(1024) void k_moe_route_plan(const float* __restrict
 extern "C" int imparo_moe_route_plan_tokens() { return MOE_ROUTE_PLAN_TOKENS; }
 
 extern "C" int imparo_moe_route_plan(const float* logits, const float* correction, int32_t* choice, float* weight,
-                                     int n_tokens, int n_router, int top, int n_experts, int tile_rows,
+                                     int n_tokens, int n_router, int top, int scoring, int n_experts, int tile_rows,
                                      int32_t* slot_of_entry, int32_t* entry_of_slot, int32_t* tiles, int max_tiles,
                                      imparo_stream stream) {
     if (!logits || !choice || !weight || !slot_of_entry || !entry_of_slot || !tiles) return IMPARO_BAD_ARGUMENT;
+    if (scoring != MOE_SCORE_SOFTMAX && scoring != MOE_SCORE_SIGMOID) return IMPARO_BAD_ARGUMENT;
     if (n_tokens < 0 || n_tokens > MOE_ROUTE_PLAN_TOKENS) return IMPARO_BAD_ARGUMENT;
     if (n_router < 1 || n_router > MOE_MAX_ROUTER || top < 1 || top > n_router || top > MOE_MAX_TOP)
         return IMPARO_BAD_ARGUMENT;
@@ -197,7 +209,7 @@ extern "C" int imparo_moe_route_plan(const float* logits, const float* correctio
     if (max_tiles < imparo_moe_max_tiles(n_tokens * top, n_experts, tile_rows)) return IMPARO_SCRATCH_TOO_SMALL;
     if (n_tokens == 0) return IMPARO_OK;
     k_moe_route_plan<<<1, 1024, 0, (hipStream_t)stream>>>(logits, correction, choice, weight, n_tokens, n_router, top,
-                                                          n_experts, tile_rows, slot_of_entry, entry_of_slot, tiles,
+                                                          scoring, n_experts, tile_rows, slot_of_entry, entry_of_slot, tiles,
                                                           max_tiles);
     return launch_status();
 }
@@ -534,6 +546,47 @@ extern "C" int imparo_moe_gemm(const void* a, int a_ld, int gather_div, const in
     return launch_status();
 }
 
+// ---------------------------------------------------------------- gated experts
+// hidden[slot, j] = silu(w g) * (w u) with g = gu[slot, j], u = gu[slot, half + j] (an expert's gate and up
+// rows stacked in one product) and w the weight of the slot's entry (null: 1): an expert without biases that
+// reads w * h has w times the products of h. Columns j >= ff (a hidden width filled up for the product
+// that follows) hold zeros in gu already and give zeros.
+template <typename TOut>
+__global__ void k_moe_gated(const float* __restrict__ gu, const float* __restrict__ weight,
+                            const int32_t* __restrict__ entry_of_slot, int n_entries, TOut* __restrict__ hidden,
+                            int half, long long total) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const long long slot = i / half;
+    const int j = (int)(i - slot * half);
+    float w = 1.0f;
+    if (weight) {
+        const int e = entry_of_slot[slot];          // a row behind the last slot names no entry
+        w = (e >= 0 && e < n_entries) ? weight[e] : 0.f;
+    }
+    const float g = w * gu[slot * 2 * half + j], u = w * gu[slot * 2 * half + half + j];
+    store_f32<TOut>(hidden, (size_t)i, g / (1.0f + expf(-g)) * u);
+}
+
+// n_slots: the entries that got a slot are the first ones of gu and hidden; where some entries have none
+// (experts past the last real one) the rows behind the last slot are computed from whatever gu holds and
+// never read.
+extern "C" int imparo_moe_gated(const float* gu, const float* weight, const int32_t* entry_of_slot, void* hidden,
+                                int out_dtype, int n_slots, int half, imparo_stream stream) {
+    if (!gu || !hidden || n_slots < 0 || half < 1 || (weight && !entry_of_slot)) return IMPARO_BAD_ARGUMENT;
+    if (n_slots == 0) return IMPARO_OK;
+    const long long total = (long long)n_slots * half;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    hipStream_t s = (hipStream_t)stream;
+    if (out_dtype == IMPARO_F32)
+        k_moe_gated<float><<<blocks, 256, 0, s>>>(gu, weight, entry_of_slot, n_slots, (float*)hidden, half, total);
+    else if (out_dtype == IMPARO_BF16)
+        k_moe_gated<bf16_t><<<blocks, 256, 0, s>>>(gu, weight, entry_of_slot, n_slots, (bf16_t*)hidden, half, total);
+    else
+        return IMPARO_BAD_ARGUMENT;
+    return launch_status();
+}
+
 // ---------------------------------------------------------------- combine
 // out[t] = sum over the token's choices, in their order, of weight * (the expert's row, or for an
 // expert past the last real one the token's input).
@@ -547,7 +600,7 @@ __global__ void k_moe_combine(const float* __restrict__ y, const T* __restrict__
     if (threadIdx.x < top) {
         const int e = choice[(size_t)t * top + threadIdx.x];
         slot[threadIdx.x] = e < n_experts ? slot_of_entry[(size_t)t * top + threadIdx.x] : -1;
-        w[threadIdx.x] = weight[(size_t)t * top + threadIdx.x];
+        w[threadIdx.x] = weight ? weight[(size_t)t * top + threadIdx.x] : 1.0f;
     }
     __syncthreads();
     for (int i = threadIdx.x; i < width; i += blockDim.x) {
@@ -563,7 +616,7 @@ __global__ void k_moe_combine(const float* __restrict__ y, const T* __restrict__
 extern "C" int imparo_moe_combine(const float* y, const void* h, int h_dtype, const int32_t* choice,
                                   const float* weight, const int32_t* slot_of_entry, float* out, int n_tokens,
                                   int width, int top, int n_experts, imparo_stream stream) {
-    if (!y || !h || !choice || !weight || !slot_of_entry || !out || n_tokens < 0 || width < 1) return IMPARO_BAD_ARGUMENT;
+    if (!y || !h || !choice || !slot_of_entry || !out || n_tokens < 0 || width < 1) return IMPARO_BAD_ARGUMENT;
     if (top < 1 || top > MOE_MAX_TOP || n_experts < 0) return IMPARO_BAD_ARGUMENT;
     if (n_tokens == 0) return IMPARO_OK;
     hipStream_t s = (hipStream_t)stream;

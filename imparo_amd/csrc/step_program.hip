@@ -427,7 +427,8 @@ extern "C" int imparo_load_code() {
     const int status[] = {imparo_load_code_attention(), imparo_load_code_attention_mfma(), imparo_load_code_decode_rows(), imparo_load_code_elementwise(),
                           imparo_load_code_gemm(),      imparo_load_code_rope_cache(),     imparo_load_code_sampling(),
                           imparo_load_code_diff_attention(), imparo_load_code_row_ops(), imparo_load_code_selective_scan(),
-                          imparo_load_code_moe()};
+                          imparo_load_code_moe(), imparo_load_code_gated_ops(), imparo_load_code_hgrn2(),
+                          imparo_load_code_latent_attention()};
     for (int s : status)
         if (s != IMPARO_OK) return s;
     return IMPARO_OK;

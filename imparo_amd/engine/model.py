@@ -14,6 +14,7 @@ import torch
 
 from ..cache.pages import StateSpec
 from ..config.plan import ModelPlan, PartSpec
+from ..kernels import ops
 from ..parts import part_class
 from ..parts.base import Declared, Residual, StepContext, emits
 
@@ -85,7 +86,14 @@ class Model:
         logits [wanted, vocab] for `want_rows` (indices into the packed
         batch), or None if nothing is wanted; the head is skipped then."""
         res = Residual(self.embedding.forward(ctx, token_ids))
+        ctx.token_ids = token_ids
+        kept = None
+        if any(call.add_input for call in self.plan.order):
+            # a run order that takes the embedding's output into the stream again keeps it apart
+            kept = self.embedding.forward(ctx, token_ids, name="embedding_kept")
         for i, call in enumerate(self.plan.order):
+            if call.add_input:
+                ops.add_rows(res.x, kept)        # (what is pending on the stream is added by the next norm, as ever)
             self.blocks[call.layer].forward(ctx, res, self.site_of_call[i], call.cache_of is None)
         if want_rows is None or want_rows.shape[0] == 0:
             return None
@@ -99,6 +107,8 @@ class Model:
         from ..kernels.program import MAX_GROUPS, Program
         if len(set(group_of_site.values())) > MAX_GROUPS:
             return None
+        if any(call.add_input for call in self.plan.order):
+            return None          # the step program does not take the embedding's output into the stream again
         blocks_emit = all(emits(b) and getattr(b, "can_emit", lambda: True)() for b in self.blocks)
         if not (blocks_emit and emits(self.embedding) and emits(self.final_norm, "emit_head", "forward_rows")
                 and getattr(self.final_norm, "can_emit", lambda: True)() and emits(self.head, "emit_projection")):

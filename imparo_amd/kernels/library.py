@@ -70,9 +70,17 @@ _SIGNATURES = {
     "imparo_embed_gather_scaled": [P, I, P, P, I, I, I, F, P],
     "imparo_qk_norm_rope_store_dv": [P, P, P, F, P, I, I, P, P, P, I, I, P, P, P, I, I, I, I, I, I, I, I, I, P],
     "imparo_attention_dv": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, I, F, I, I, P],
-    "imparo_moe_route": [P, P, P, P, I, I, I, P],
+    "imparo_moe_route": [P, P, P, P, I, I, I, I, P],
+    "imparo_moe_gated": [P, P, P, P, I, I, I, P],
+    "imparo_attention_latent": [P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P],
+    "imparo_latent_store": [P, P, P, F, P, I, I, P, P, P, I, I, I, P, P, P, I, I, I, I, I, I, P],
+    "imparo_head_gemm": [P, I, I, P, I, P, I, I, I, I, I, I, I, P],
+    "imparo_hgrn2_scan": [P, I, I, I, I, P, P, P, P, P, P, I, I, I, I, P],
+    "imparo_gated_sum": [P, P, P, P, I, P, I, I, I, P],
+    "imparo_side_gate": [P, P, I, I, I, P, I, P, I, I, I, I, P],
+    "imparo_add_rows": [P, P, c_int64, P],
     "imparo_moe_route_plan_tokens": [],
-    "imparo_moe_route_plan": [P, P, P, P, I, I, I, I, I, P, P, P, I, P],
+    "imparo_moe_route_plan": [P, P, P, P, I, I, I, I, I, I, P, P, P, I, P],
     # x, y, h, h_dtype, choice, weight, slot_of_entry, top, n_experts, n_rows_x, rows, w_post, eps_post, w_next, eps_next,
     # out, out_dtype, n_out, width, stream
     "imparo_post_norm_add_moe": [P, P, P, I, P, P, P, I, I, I, P, P, F, P, F, P, I, I, I, P],

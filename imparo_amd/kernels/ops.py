@@ -14,6 +14,8 @@ import torch
 from .library import library
 
 F32, BF16 = 0, 1
+ATTENTION_MAX_HEAD_DIM = 576      # the wave attention kernel's longest key row
+HGRN2_MAX_DIM = 256               # state rows a head of the gated linear recurrence
 _CODES = {torch.float32: F32, torch.bfloat16: BF16}
 
 
@@ -751,17 +753,35 @@ def diff_attention_tiles(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.
 
 # ---------------------------------------------------------------- routed feed-forward, norm on a sublayer's result
 MOE_EPILOGUES = {None: 0, "none": 0, "relu2": 1}
+MOE_SCORINGS = {"softmax": 0, "sigmoid": 1}
 
 
 def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], choice: torch.Tensor, weight: torch.Tensor,
-              top: int) -> None:
-    """choice[t] = the `top` router outputs with the largest softmax(logits[t]) + correction, weight[t] their
-    softmax scores (as they are)."""
+              top: int, scoring: str = "softmax") -> None:
+    """choice[t] = the `top` router outputs with the largest score + correction, weight[t] their scores (as
+    they are); scores are softmax(logits[t]) or, with scoring "sigmoid", the sigmoid of each output."""
     n, r = logits.shape
     _check(library().imparo_moe_route(
         _dev(logits, "router logits", torch.float32), _dev(correction, "router correction", torch.float32, (r,)),
         _dev(choice, "choice", torch.int32, (n, top)), _dev(weight, "choice weights", torch.float32, (n, top)),
-        n, r, top, _stream()), "moe_route")
+        n, r, top, MOE_SCORINGS[scoring], _stream()), "moe_route")
+
+
+def moe_gated(gu: torch.Tensor, weight: Optional[torch.Tensor], entry_of_slot: Optional[torch.Tensor],
+              hidden: torch.Tensor) -> torch.Tensor:
+    """hidden[slot, j] = silu(w g) * (w u) with g = gu[slot, j], u = gu[slot, half + j] and w the weight of the
+    slot's entry (weight None: 1)."""
+    n, two = gu.shape
+    half = two // 2
+    if two != 2 * half or tuple(hidden.shape) != (n, half):
+        raise KernelArgumentError(f"moe_gated: gu is {tuple(gu.shape)}, hidden {tuple(hidden.shape)}")
+    if weight is not None and (entry_of_slot is None or weight.numel() < n or entry_of_slot.numel() < n):
+        raise KernelArgumentError("moe_gated: a weight and an entry per slot are needed")
+    _check(library().imparo_moe_gated(
+        _dev(gu, "gate and up products", torch.float32), _dev(weight, "choice weights", torch.float32),
+        _dev(entry_of_slot, "entry_of_slot", torch.int32), _dev(hidden, "hidden"), _code(hidden, "hidden"),
+        n, half, _stream()), "moe_gated")
+    return hidden
 
 
 def moe_route_plan_tokens() -> int:
@@ -771,7 +791,7 @@ def moe_route_plan_tokens() -> int:
 
 def moe_route_plan(logits: torch.Tensor, correction: Optional[torch.Tensor], choice: torch.Tensor, weight: torch.Tensor,
                    top: int, n_experts: int, tile_rows: int, slot_of_entry: torch.Tensor, entry_of_slot: torch.Tensor,
-                   tiles: torch.Tensor) -> None:
+                   tiles: torch.Tensor, scoring: str = "softmax") -> None:
     """`moe_route` and `moe_plan` in one launch, for the few tokens of a decode step."""
     n, r = logits.shape
     _dev(slot_of_entry, "slot_of_entry", torch.int32, (n * top,))
@@ -779,7 +799,7 @@ def moe_route_plan(logits: torch.Tensor, correction: Optional[torch.Tensor], cho
     _check(library().imparo_moe_route_plan(
         _dev(logits, "router logits", torch.float32), _dev(correction, "router correction", torch.float32, (r,)),
         _dev(choice, "choice", torch.int32, (n, top)), _dev(weight, "choice weights", torch.float32, (n, top)),
-        n, r, top, n_experts, tile_rows, slot_of_entry.data_ptr(), entry_of_slot.data_ptr(),
+        n, r, top, MOE_SCORINGS[scoring], n_experts, tile_rows, slot_of_entry.data_ptr(), entry_of_slot.data_ptr(),
         _dev(tiles, "tiles", torch.int32), tiles.shape[0], _stream()), "moe_route_plan")
 
 
@@ -823,8 +843,10 @@ def moe_gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, tiles: torch.T
     return out
 
 
-def moe_combine(y: torch.Tensor, h: torch.Tensor, choice: torch.Tensor, weight: torch.Tensor,
+def moe_combine(y: torch.Tensor, h: torch.Tensor, choice: torch.Tensor, weight: Optional[torch.Tensor],
                 slot_of_entry: torch.Tensor, n_experts: int, out: torch.Tensor) -> torch.Tensor:
+    """out[t] = the sum over a token's choices of weight * (its expert's row, or h[t] for an expert past the
+    last real one); weight None: every weight is 1."""
     n, top = choice.shape
     width = h.shape[1]
     _check(library().imparo_moe_combine(
@@ -846,6 +868,8 @@ def post_norm_add(x: torch.Tensor, delta, w_post: torch.Tensor, eps_post: float,
     n_out = n_x if rows is None else rows.shape[0]
     if not isinstance(delta, torch.Tensor):
         top = delta.choice.shape[1]
+        if delta.weight is None:
+            raise KernelArgumentError("post_norm_add: the experts' sum inside this launch needs the choice's weights")
         if w_next is not None and (out is None or tuple(out.shape) != (n_out, width)):
             raise KernelArgumentError("post_norm_add: the next norm needs an output of one row per taken row")
         if w_next is None and rows is not None:
@@ -874,3 +898,114 @@ def post_norm_add(x: torch.Tensor, delta, w_post: torch.Tensor, eps_post: float,
         _dev(out, "normed") if w_next is not None else None, _code(out, "normed") if w_next is not None else 0,
         n_out, width, _stream()), "post_norm_add")
     return out
+
+
+# ---------------------------------------------------------------- attention over a cached latent
+def latent_store(q_rows: torch.Tensor, kv_rows: torch.Tensor, norm_weight: torch.Tensor, eps: float,
+                 inv_freq: Optional[torch.Tensor], interleaved: bool, positions: torch.Tensor, row_of_token: torch.Tensor,
+                 block_table: Optional[torch.Tensor], page_size: int, cache: Optional[torch.Tensor], q_plain: torch.Tensor,
+                 q_full: torch.Tensor, heads: int, dim: int, rot_dim: int, rank: int) -> None:
+    """The latent's norm, the rotation of the shared key part and of every head's rotated query part, the write
+    of [latent | rotated key part] into the token's page, and the queries laid out for the absorbed products."""
+    n = q_rows.shape[0]
+    n_freq = 0 if inv_freq is None else inv_freq.shape[0]
+    n_pages = table_stride = 0
+    if cache is not None:
+        n_pages = cache.shape[0]
+        _dev(cache, "latent cache", q_full.dtype, (n_pages, page_size, rank + rot_dim))
+        if block_table is None or block_table.dim() != 2:
+            raise KernelArgumentError("latent_store: a [rows, pages] block table is needed to write the cache")
+        table_stride = block_table.shape[1]
+    _check(library().imparo_latent_store(
+        _dev(q_rows, "query rows", torch.float32, (n, heads * (dim + rot_dim))),
+        _dev(kv_rows, "latent rows", torch.float32, (n, rank + rot_dim)),
+        _dev(norm_weight, "latent norm weight", torch.float32, (rank,)), float(eps),
+        _dev(inv_freq, "inverse frequencies", torch.float32), n_freq, int(interleaved),
+        _dev(positions, "positions", torch.int32, (n,)), _dev(row_of_token, "row_of_token", torch.int32, (n,)),
+        _dev(block_table, "block table", torch.int32), table_stride, page_size, n_pages, _dev(cache, "latent cache"),
+        _dev(q_plain, "unrotated queries", q_full.dtype, (n, heads, dim)),
+        _dev(q_full, "queries", None, (n, heads, rank + rot_dim)), _code(q_full, "queries"),
+        n, heads, dim, rot_dim, rank, _stream()), "latent_store")
+
+
+def head_gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, out_columns: Optional[int] = None) -> torch.Tensor:
+    """out[t, h, :n] = W[h] x[t, h, :] with w [heads, k, n] (an up-projection of its own per head); x [tokens,
+    heads, k]; out [tokens, heads, n], or wider rows a head of which the first n columns are written."""
+    T, H, K = x.shape
+    Hw, Kw, N = w.shape
+    if (Hw, Kw) != (H, K) or x.dtype != w.dtype:
+        raise KernelArgumentError(f"head_gemm: x is {tuple(x.shape)} {x.dtype}, the weights {tuple(w.shape)} {w.dtype}")
+    if out.dim() != 3 or out.shape[0] != T or out.shape[1] != H or out.shape[2] < N:
+        raise KernelArgumentError(f"head_gemm: out is {tuple(out.shape)}; [{T}, {H}, at least {N}] is needed")
+    _check(library().imparo_head_gemm(
+        _dev(x, "head_gemm x"), H * K, K, _dev(w, "head_gemm weights"), _code(x, "head_gemm x"),
+        _dev(out, "head_gemm out"), _code(out, "head_gemm out"), H * out.shape[2], out.shape[2], T, H, K, N, _stream()),
+        "head_gemm")
+    return out
+
+
+def attention_latent(q: torch.Tensor, cache: torch.Tensor, out: torch.Tensor, positions: torch.Tensor,
+                     row_of_token: torch.Tensor, block_table: torch.Tensor, value_dim: int, scale: float,
+                     window: Optional[int]) -> torch.Tensor:
+    """Attention in which all heads read the same cached rows: a key is a whole row, its value the row's
+    first `value_dim` numbers. One wave per (token, head); float32 or bfloat16."""
+    n, heads, row_dim = q.shape
+    n_pages, page_size, rd = cache.shape
+    if rd != row_dim or value_dim > row_dim:
+        raise KernelArgumentError(f"attention_latent: q has rows of {row_dim}, the cache of {rd}, values of {value_dim}")
+    _check(library().imparo_attention_latent(
+        _dev(q, "q"), _dev(cache, "latent cache", q.dtype), _dev(out, "attention out", q.dtype, (n, heads * value_dim)),
+        _code(q, "q"), _dev(positions, "positions", torch.int32, (n,)), _dev(row_of_token, "row_of_token", torch.int32, (n,)),
+        _dev(block_table, "block table", torch.int32), block_table.shape[1], page_size, n, heads, row_dim, value_dim,
+        n_pages, float(scale), int(window or 0), _stream()), "attention_latent")
+    return out
+
+
+# ---------------------------------------------------------------- gated linear recurrence
+def hgrn2_scan(rows: torch.Tensor, q_off: int, f_off: int, v_off: int, lower: torch.Tensor, state: torch.Tensor,
+               seg_start: torch.Tensor, seg_len: torch.Tensor, slot: torch.Tensor, out: torch.Tensor, heads: int,
+               dim: int, vdim: int) -> torch.Tensor:
+    """Per request and head, token by token: S <- diag(f) S + (1 - f) v^T, out = S^T q with q = silu(zq),
+    f = lower + (1 - lower) sigmoid(zf); rows holds zq, zf, v at the given columns."""
+    n, ld = rows.shape
+    R = seg_start.shape[0]
+    _check(library().imparo_hgrn2_scan(
+        _dev(rows, "recurrence inputs", torch.float32), ld, q_off, f_off, v_off,
+        _dev(lower, "lower bounds", torch.float32, (heads * dim,)),
+        _dev(state, "recurrent state", torch.float32, (state.shape[0], heads, dim, vdim)),
+        _dev(seg_start, "seg_start", torch.int32, (R,)), _dev(seg_len, "seg_len", torch.int32, (R,)),
+        _dev(slot, "slot", torch.int32, (R,)), _dev(out, "recurrence out", torch.float32, (n, heads * vdim)),
+        R, heads, dim, vdim, _stream()), "hgrn2_scan")
+    return out
+
+
+# ---------------------------------------------------------------- a parallel block's elementwise pieces
+def gated_sum(x: torch.Tensor, a: torch.Tensor, b: Optional[torch.Tensor], gates: torch.Tensor,
+              copy: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x += a * sigmoid(gates[:, :width]) (+ b * sigmoid(gates[:, width:])); `copy` also receives the new x."""
+    n, width = x.shape
+    _check(library().imparo_gated_sum(
+        _dev(x, "stream", torch.float32), _dev(a, "first sublayer's result", torch.float32, (n, width)),
+        _dev(b, "second sublayer's result", torch.float32, (n, width)),
+        _dev(gates, "gates", torch.float32, (n, 2 * width if b is not None else gates.shape[1])), gates.shape[1],
+        _dev(copy, "stream copy", None, (n, width)), _code(copy, "stream copy") if copy is not None else 0,
+        n, width, _stream()), "gated_sum")
+    return x
+
+
+def side_gate(z: torch.Tensor, table: torch.Tensor, offset: int, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t, j] = gelu_tanh(z[t, j]) * table[ids[t], offset + j]; columns beyond z's width become zero."""
+    n, dim = z.shape
+    vocab, table_ld = table.shape
+    _check(library().imparo_side_gate(
+        _dev(z, "side gate", torch.float32), _dev(table, "side table"), _code(table, "side table"), table_ld, offset,
+        _dev(ids, "token ids", torch.int32, (n,)), vocab, _dev(out, "gated side input", None, (n, out.shape[1])),
+        _code(out, "gated side input"), n, dim, out.shape[1], _stream()), "side_gate")
+    return out
+
+
+def add_rows(x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+    """x += y, both float32 of one shape."""
+    _check(library().imparo_add_rows(_dev(x, "x", torch.float32), _dev(y, "y", torch.float32, tuple(x.shape)),
+                                     x.numel(), _stream()), "add_rows")
+    return x

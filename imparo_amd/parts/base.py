@@ -112,6 +112,8 @@ class StepContext:
     # The float32 residual stream while a block runs the part whose result goes into it, with nothing pending
     # on it: the part may add its result there itself and return the stream instead of a delta. None: return a delta.
     stream: Optional[torch.Tensor] = None
+    # The step's token ids (int32, one a token), for a part that looks a token up in a table of its own.
+    token_ids: Optional[torch.Tensor] = None
 
     def paged(self, site: int):
         """The site's paged arrays by name, and the block table of its group."""

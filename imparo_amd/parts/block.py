@@ -16,6 +16,7 @@ from typing import Dict
 import torch
 
 from ..cache.pages import with_fixed_arrays
+from ..kernels import ops
 from .base import Residual, StepContext, emits
 from .registry import register_part
 
@@ -113,5 +114,53 @@ class SandwichBlock(PreNormBlock):
         return False          # the step program knows the pre-norm block only
 
 
+class ParallelBlock:
+    """x += gate_a * mixer(h) + gate_b * ffn(h) with h = norm(x): one norm feeds both sublayers, and each
+    result is multiplied by sigmoid(W h + b) of that same input (`mixer_gate`, `ffn_gate`: both gates are
+    one projection). Optional parts: `ffn` with `ffn_gate` (a layer may have no feed-forward), and `side`, a
+    per-layer input from the token itself that reads the stream behind the sum; its result is left pending on
+    the stream together with its norm, so that the next norm, whichever block it belongs to, applies it,
+    adds and norms the sum in one launch."""
+    role = "block"
+    graph_safe = True     # launches kernels only: a step made of such parts can be captured
+
+    def __init__(self, parts: Dict[str, object]):
+        from .gate import SigmoidGate
+        self.parts = parts
+        self.mixer_norm, self.mixer, self.mixer_gate = parts["mixer_norm"], parts["mixer"], parts["mixer_gate"]
+        self.ffn, self.ffn_gate = parts.get("ffn"), parts.get("ffn_gate")
+        self.side = parts.get("side")
+        if (self.ffn is None) != (self.ffn_gate is None):
+            raise ValueError("a block has a feed-forward and its gate, or neither")
+        self.gates = SigmoidGate.together([self.mixer_gate] + ([self.ffn_gate] if self.ffn is not None else []))
+
+    def cache_spec(self, page_size: int):
+        return self.mixer.cache_spec(page_size)
+
+    def forward(self, ctx: StepContext, res: Residual, site: int, owns_cache: bool) -> None:
+        # the norm's output once per dtype its readers ask for (one, unless some projection's sizes keep it in float32)
+        normed = {}
+
+        def h_in(dtype):
+            if dtype not in normed:
+                normed[dtype] = self.mixer_norm.forward(ctx, res, dtype, name=f"normed_{len(normed)}" if normed else "normed")
+            return normed[dtype]
+
+        h = h_in(self.mixer.in_dtype)
+        gates = self.gates(ctx, h_in(self.gates.in_dtype), torch.float32, "gates")
+        m = self.mixer.forward(ctx, site, owns_cache, h)
+        f = None if self.ffn is None else self.ffn.forward(ctx, h_in(self.ffn.in_dtype))
+        copy = None
+        if self.side is not None:
+            copy = ctx.workspace.get("stream_copy", tuple(res.x.shape), self.side.in_dtype)
+        ops.gated_sum(res.x, m, f, gates, copy)
+        if self.side is not None:
+            res.pending, res.post = self.side.forward(ctx, copy), self.side.as_post()
+
+    def can_emit(self) -> bool:
+        return False          # the step program knows the pre-norm block only
+
+
 register_part("block", "pre_norm", PreNormBlock)
+register_part("block", "parallel", ParallelBlock)
 register_part("block", "sandwich", SandwichBlock)

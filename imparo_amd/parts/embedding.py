@@ -6,7 +6,8 @@ head (logits = W h for the rows that want logits, no bias, no softcap:
 `tensor` names the table outright where a checkpoint does not call it
 `<prefix>.weight`. The sinusoidal embedding adds a position vector to the
 gathered row: entry 2i is sin(p * base^(-2i/width)), entry 2i+1 the cosine of
-the same angle, angles in float32."""
+the same angle, angles in float32. `norm` (the spec of a norm part) norms the
+gathered rows before they become the stream."""
 from __future__ import annotations
 
 from typing import Dict
@@ -19,7 +20,7 @@ from ..kernels import ops
 from ..weights.loader import TensorDecl
 from .base import Declared, StepContext
 from .linear import Linear, place_matrix, place_projection
-from .registry import register_part
+from .registry import part_class, register_part
 
 
 def _table_name(spec: PartSpec) -> str:
@@ -32,7 +33,11 @@ class Embedding:
 
     @staticmethod
     def declare(spec: PartSpec) -> Declared:
-        return {_table_name(spec): (TensorDecl((spec["vocab"], spec["width"])), "matrix")}
+        out = {_table_name(spec): (TensorDecl((spec["vocab"], spec["width"])), "matrix")}
+        norm = spec.get("norm")
+        if norm is not None:
+            out.update(part_class("norm", norm.kind).declare(norm))
+        return out
 
     def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], device: torch.device,
                  engine_dtype: torch.dtype, placed: Dict[str, torch.Tensor]):
@@ -42,13 +47,23 @@ class Embedding:
         self.table = placed[name]
         self.vocab, self.width = spec["vocab"], spec["width"]
         self.scale = float(spec.get("scale", 1.0))
+        norm = spec.get("norm")
+        self.norm = None if norm is None else part_class("norm", norm.kind)(norm, tensors, device, engine_dtype)
+        if self.norm is not None and getattr(self.norm, "groups", 1) != 1:
+            raise ValueError("the norm on the embedding's rows does not cut them into groups")
 
-    def forward(self, ctx: StepContext, token_ids: torch.Tensor) -> torch.Tensor:
-        x = ctx.workspace.get("residual", (token_ids.shape[0], self.width), torch.float32)
-        return ops.embed_gather(self.table, token_ids, x, self.scale)
+    def forward(self, ctx: StepContext, token_ids: torch.Tensor, name: str = "residual") -> torch.Tensor:
+        """The rows of the stream, float32, in the workspace buffer `name` (a caller that needs the
+        embedding's output twice, once to keep, asks twice: the same launches, the same bits)."""
+        x = ctx.workspace.get(name, (token_ids.shape[0], self.width), torch.float32)
+        if self.norm is None:
+            return ops.embed_gather(self.table, token_ids, x, self.scale)
+        raw = ctx.workspace.get("embedding_rows", (token_ids.shape[0], self.width), torch.float32)
+        ops.embed_gather(self.table, token_ids, raw, self.scale)
+        return ops.rms_norm(raw, self.norm.weight, self.norm.eps, x)
 
     def can_emit(self) -> bool:
-        return self.scale == 1.0          # the step program's gather has no scale
+        return self.scale == 1.0 and self.norm is None     # the step program's gather has neither
 
     def emit(self, program) -> None:
         """Appends `forward` to a native step program."""

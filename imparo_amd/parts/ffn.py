@@ -34,21 +34,23 @@ class SwiGlu:
     @classmethod
     def declare(cls, spec: PartSpec) -> Declared:
         n = cls._names(spec)
+        sfx = spec.get("weight_suffix", ".weight")
         E, F = spec["width"], spec["hidden"]
         return {
-            n["gate"] + ".weight": (TensorDecl((F, E)), "matrix"),
-            n["up"] + ".weight": (TensorDecl((F, E)), "matrix"),
-            n["down"] + ".weight": (TensorDecl((E, F)), "matrix"),
+            n["gate"] + sfx: (TensorDecl((F, E)), "matrix"),
+            n["up"] + sfx: (TensorDecl((F, E)), "matrix"),
+            n["down"] + sfx: (TensorDecl((E, F)), "matrix"),
         }
 
     def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], device: torch.device,
                  engine_dtype: torch.dtype):
         n = self._names(spec)
+        sfx = spec.get("weight_suffix", ".weight")          # what a checkpoint appends to a matrix's name
         self.width, self.hidden = spec["width"], spec["hidden"]
-        gate, up = tensors[n["gate"] + ".weight"], tensors[n["up"] + ".weight"]
+        gate, up = tensors[n["gate"] + sfx], tensors[n["up"] + sfx]
         if gate.dtype != up.dtype:
             gate, up = gate.to(torch.float32), up.to(torch.float32)
-        down = tensors[n["down"] + ".weight"]
+        down = tensors[n["down"] + sfx]
         # The bfloat16 kernels walk K in steps of 8. A hidden width that is no multiple of 8 is
         # filled up with hidden units whose weights are zero: silu(0) * 0 = 0 goes through zero
         # columns of the way back, so every sum is the one it was.
@@ -60,7 +62,7 @@ class SwiGlu:
         # gate and up as one projection with alternating rows (g0, u0, g1, u1, ...): the same dot
         # products, one launch, and the GEMM's epilogue applies silu(gate) * up before it stores
         fused = torch.stack([gate, up], dim=1).reshape(2 * gate.shape[0], self.width)
-        self.gate_up = Linear(place_matrix(fused, engine_dtype, device))
+        self.gate_up = Linear(place_projection(fused, engine_dtype, device))
         self.down = Linear(place_matrix(down, engine_dtype, device))
 
     @property

@@ -10,9 +10,14 @@ experts that pass their input through. The result is the weighted sum of the
 chosen experts' outputs, added in the order of the choice.
 
 Parameters: width, hidden (an expert's), experts, identity, top, activation
-("relu2": the square of max(z, 0)), and the tensors' names: `router`,
-`correction` (None: no correction), `expert_up` / `expert_down` as patterns
-with `{e}` for the expert's number.
+("relu2": the square of max(z, 0); "swiglu": a gated expert, y = Wdown
+(silu(Wgate n) * (Wup n)), whose gate matrix is named by `expert_gate`),
+scoring ("softmax" over all router outputs, or "sigmoid" of each output by
+itself), weigh ("output": a chosen expert's result is multiplied by its
+weight; "input": the expert reads its input times its weight and the results
+are added as they are), and the tensors' names: `router`, `correction` (None:
+no correction), `expert_up` / `expert_down` as patterns with `{e}` for the
+expert's number.
 
 The experts' matrices lie stacked, [experts, out, in]. A step sorts its (token,
 choice) entries by expert on the device and runs the two products over tiles of
@@ -39,7 +44,8 @@ class RoutedExperts:
 
     @staticmethod
     def _names(spec: PartSpec) -> Dict[str, str]:
-        names = dict(router="router", correction="correction", expert_up="e{e}.up", expert_down="e{e}.down")
+        names = dict(router="router", correction="correction", expert_up="e{e}.up", expert_down="e{e}.down",
+                     expert_gate="e{e}.gate")
         names.update(spec.get("names") or {})
         return {k: (None if v is None else f"{spec.prefix}.{v}") for k, v in names.items()}
 
@@ -51,6 +57,8 @@ class RoutedExperts:
         if n["correction"] is not None:
             out[n["correction"]] = (TensorDecl((X + I,), "vector"), "bias")
         for e in range(X):
+            if spec.get("activation", "relu2") == "swiglu":
+                out[n["expert_gate"].format(e=e)] = (TensorDecl((F, E)), "matrix")
             out[n["expert_up"].format(e=e)] = (TensorDecl((F, E)), "matrix")
             out[n["expert_down"].format(e=e)] = (TensorDecl((E, F)), "matrix")
         return out
@@ -61,8 +69,18 @@ class RoutedExperts:
         self.width, self.hidden = spec["width"], spec["hidden"]
         self.experts, self.identity, self.top = spec["experts"], int(spec.get("identity", 0)), spec["top"]
         self.activation = spec.get("activation", "relu2")
-        if self.activation not in ops.MOE_EPILOGUES or self.activation in (None, "none"):
+        self.gated = self.activation == "swiglu"
+        if not self.gated and (self.activation not in ops.MOE_EPILOGUES or self.activation in (None, "none")):
             raise ValueError(f"the experts' activation {self.activation!r} is not one the product's epilogue knows")
+        self.scoring = spec.get("scoring", "softmax")
+        if self.scoring not in ops.MOE_SCORINGS:
+            raise ValueError(f"the router's scoring {self.scoring!r} is none of {sorted(ops.MOE_SCORINGS)}")
+        self.weigh = spec.get("weigh", "output")
+        if self.weigh not in ("output", "input"):
+            raise ValueError(f"weigh is 'output' or 'input', got {self.weigh!r}")
+        if self.weigh == "input" and (not self.gated or self.identity):
+            # w act(W n) = act(W (w n)) holds for no activation here but the gated one's kernel, which takes w itself
+            raise ValueError("experts that read their input times their weight are the gated ones, without pass-through experts")
         if not 1 <= self.top <= self.experts + self.identity:
             raise ValueError(f"{self.top} of {self.experts + self.identity} experts cannot be chosen")
         # bfloat16 x bfloat16 products are exact in float32 and the sums are float32: the router runs in 32 bits
@@ -71,14 +89,21 @@ class RoutedExperts:
         self.correction = None if n["correction"] is None else place_vector(tensors[n["correction"]], device)
         ups = [tensors[n["expert_up"].format(e=e)] for e in range(self.experts)]
         downs = [tensors[n["expert_down"].format(e=e)] for e in range(self.experts)]
+        gates = [tensors[n["expert_gate"].format(e=e)] for e in range(self.experts)] if self.gated else []
         if self.experts:
             up, down = torch.stack(ups), torch.stack(downs)
+            gate = torch.stack(gates) if self.gated else None
             # The bfloat16 products walk K in steps of 8: a hidden width that is no multiple of 8 is filled up
             # with hidden units of zero weight (act(0) = 0 goes through zero columns of the way back).
             fill = (-self.hidden) % 8
             if fill and engine_dtype != torch.float32:
                 up = torch.cat([up, up.new_zeros(self.experts, fill, self.width)], dim=1)
                 down = torch.cat([down, down.new_zeros(self.experts, self.width, fill)], dim=2)
+                if self.gated:
+                    gate = torch.cat([gate, gate.new_zeros(self.experts, fill, self.width)], dim=1)
+            if self.gated:
+                # an expert's gate rows, then its up rows: one product makes both, a launch behind it gates
+                up = torch.cat([gate.to(up.dtype), up], dim=1)
             if engine_dtype != torch.float32 and (self.width % 8 or self.router.in_dtype == torch.float32):
                 up, down = up.to(torch.float32), down.to(torch.float32)      # such a width runs in float32 throughout
             self.up = place_matrix(up, engine_dtype, device)
@@ -106,16 +131,23 @@ class RoutedExperts:
             tiles = ws.get("moe_tiles", (ops.moe_max_tiles(entries, X, rows), 3), torch.int32)
             entry_of_slot = ws.get("moe_entry_of_slot", (entries,), torch.int32)
             if T <= ops.moe_route_plan_tokens():      # a decode step: choice and plan in one launch
-                ops.moe_route_plan(z, self.correction, choice, weight, top, X, rows, slot_of_entry, entry_of_slot, tiles)
+                ops.moe_route_plan(z, self.correction, choice, weight, top, X, rows, slot_of_entry, entry_of_slot, tiles,
+                                   scoring=self.scoring)
             else:
-                ops.moe_route(z, self.correction, choice, weight, top)
+                ops.moe_route(z, self.correction, choice, weight, top, scoring=self.scoring)
                 ops.moe_plan(choice, X, rows, slot_of_entry, entry_of_slot, tiles)
-            hidden = ws.get("moe_hidden", (entries, self.up.shape[1]), self.up.dtype, alias="mixer_in")
-            ops.moe_gemm(n, self.up, hidden, tiles, rows, entry_of_slot, gather_div=top, epilogue=self.activation)
+            if self.gated:
+                both = ws.get("moe_gate_up", (entries, self.up.shape[1]), torch.float32, alias="mixer_in")
+                ops.moe_gemm(n, self.up, both, tiles, rows, entry_of_slot, gather_div=top)
+                hidden = ws.get("moe_hidden", (entries, self.up.shape[1] // 2), self.down.dtype)
+                ops.moe_gated(both, weight.view(-1) if self.weigh == "input" else None, entry_of_slot, hidden)
+            else:
+                hidden = ws.get("moe_hidden", (entries, self.up.shape[1]), self.up.dtype, alias="mixer_in")
+                ops.moe_gemm(n, self.up, hidden, tiles, rows, entry_of_slot, gather_div=top, epilogue=self.activation)
             ops.moe_gemm(hidden, self.down, y, tiles, rows)
         else:
-            ops.moe_route(z, self.correction, choice, weight, top)
-        return RowsToCombine(y, n, choice, weight, slot_of_entry, X)
+            ops.moe_route(z, self.correction, choice, weight, top, scoring=self.scoring)
+        return RowsToCombine(y, n, choice, None if self.weigh == "input" else weight, slot_of_entry, X)
 
     def forward(self, ctx: StepContext, n: torch.Tensor) -> torch.Tensor:
         r = self.forward_rows(ctx, n)

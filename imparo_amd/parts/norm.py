@@ -10,7 +10,9 @@ each is divided by its own root mean square; the weight spans the whole row.
 distance from one). `scale_tensor` names a second vector of the row's width and
 `multiplier` a constant that the normed row is multiplied by as well (a layer
 scale and a residual multiplier on a norm that sits behind a sublayer): all
-three are folded into one float32 weight when the model is loaded.
+three are folded into one float32 weight when the model is loaded. `scalar`: the
+stored weight is a single number for the whole row (a tensor without
+dimensions), spread over the row's width when the model is loaded.
 
 A block may leave its sublayer's result pending on the stream together with
 the norm it goes through before the add (`Residual.post`); this norm then
@@ -40,7 +42,8 @@ class RmsNorm:
     @classmethod
     def declare(cls, spec: PartSpec) -> Declared:
         # a weight that an offset of 1 is added to is drawn near zero
-        out = {cls._tensor(spec): (TensorDecl((spec["width"],), "vector"), "bias" if spec.get("offset") else "norm")}
+        shape = () if spec.get("scalar") else (spec["width"],)
+        out = {cls._tensor(spec): (TensorDecl(shape, "vector"), "bias" if spec.get("offset") else "norm")}
         if spec.get("scale_tensor"):
             out[spec["scale_tensor"]] = (TensorDecl((spec["width"],), "vector"), "norm")
         return out
@@ -53,6 +56,8 @@ class RmsNorm:
         if self.groups < 1 or self.width % self.groups:
             raise ValueError(f"a norm over {self.width} values cannot be cut into {self.groups} equal parts")
         weight = tensors[self._tensor(spec)].to(torch.float32) + float(spec.get("offset") or 0.0)
+        if spec.get("scalar"):
+            weight = weight.reshape(1).expand(self.width)
         if spec.get("scale_tensor"):
             weight = weight * tensors[spec["scale_tensor"]].to(torch.float32)
         if spec.get("multiplier") is not None:

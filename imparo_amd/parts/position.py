@@ -58,6 +58,11 @@ class RopeNeox:
         self.inv_freq: Optional[torch.Tensor] = torch.from_numpy(inv).to(device)
 
 
+class RopePairs(RopeNeox):
+    """The same table with neighbouring dimensions as pairs: pair i is dims (2i, 2i + 1)."""
+    interleaved = True
+
+
 class NoPosition:
     """No rotation: keys are cached as the norm leaves them."""
     role = "position"
@@ -70,4 +75,5 @@ class NoPosition:
 
 
 register_part("position", "rope_neox", RopeNeox)
+register_part("position", "rope_pairs", RopePairs)
 register_part("position", "none", NoPosition)

@@ -1,12 +1,12 @@
 """Registries of parts: one per role (norm, position, mixer, feed_forward,
-block, embedding, head, shift). A plan's PartSpec.kind picks the class; anything
+block, embedding, head, shift, gate, side). A plan's PartSpec.kind picks the class; anything
 registered here, by the framework or by a user, can appear in a plan.
 """
 from __future__ import annotations
 
 from typing import Dict
 
-ROLES = ("norm", "position", "mixer", "feed_forward", "block", "embedding", "head", "shift")
+ROLES = ("norm", "position", "mixer", "feed_forward", "block", "embedding", "head", "shift", "gate", "side")
 _PARTS: Dict[str, Dict[str, type]] = {role: {} for role in ROLES}
 
 

@@ -5,7 +5,8 @@ so the folder does not depend on the order tensors are declared in. The
 distributions: matrices and embeddings N(0, 0.02); depthwise conv taps
 N(0, 0.1); norm weights 1 + U(-0.1, 0.1); biases N(0, 0.02); a few numbers
 of a layer that act as they are (an activation's coefficients, the logarithms
-of decays: "wide") N(0, 0.5).
+of decays: "wide") N(0, 0.5); numbers that must lie between 0 and 1 (a gate's
+lower bound: "unit") U(0, 0.9).
 """
 from __future__ import annotations
 
@@ -32,6 +33,8 @@ def random_tensor(seed: int, name: str, decl: TensorDecl, init: str) -> torch.Te
     g = _generator(seed, name)
     if init == "norm":
         return 1.0 + (torch.rand(decl.shape, generator=g) * 0.2 - 0.1)
+    if init == "unit":
+        return torch.rand(decl.shape, generator=g) * 0.9
     std = {"conv": 0.1, "wide": 0.5}.get(init, 0.02)
     return torch.randn(decl.shape, generator=g) * std
 
