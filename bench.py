@@ -418,16 +418,40 @@ def pupalorn_shape(width, heads, kv_heads, expert_ff, experts=8, top=4, identity
                 embedding=dict(scale=1.0), layers=[dict(type="attention", mixer=mixer(i), mlp=mlp) for i in range(layers)])
 
 
-def compare_workload(workload, sizes, dtype, steps, warmup):
-    """Prefill and decode throughput of one design at some sizes, beside LFM2 (the closest model the engine
-    has) at equal layer sizes, through the same loops. `sizes`: (name, LFM2 configuration, the design's)."""
+def kosalorn_shape(width, heads, expert_ff, dense_ff, experts=8, top=4, layers=16, window=4096):
+    """A Kosalorn model with as many heads and as wide values as the Pupalorn shape above (heads of 64 unrotated and
+    32 rotated numbers, values of 64, a cached latent of width / 8 beside the 32 rotated ones), in a run of four
+    layers: attention with a window and queries through a latent, causal attention with direct queries, attention
+    with a window over a dense feed-forward, and the gated recurrence (heads of 128 by 128). Gated experts of
+    three matrices each, `top` of `experts` a token; a per-layer token input of 32 numbers."""
+    rank = width // 8
+    def attention(kind, windowed):
+        m = dict(heads=heads, dim=64, rot_dim=32, vdim=64, kv_rank=rank, scale=96 ** -0.5,
+                 rot=dict(dims=32, base=1000000.0))
+        if kind == "latent_attention":
+            m["q_rank"] = 3 * width // 8
+        if windowed:
+            m["mask"] = dict(size=window)
+        return dict(type=kind, mixer=m)
+    moe = dict(kind="moe", expert=dict(ff=expert_ff), router=dict(experts=experts, top=top))
+    run = [dict(attention("latent_attention", True), mlp=moe), dict(attention("latent_attention_2", False), mlp=moe),
+           dict(attention("latent_attention", True), mlp=dict(kind="dense", ff=dense_ff)),
+           dict(type="hgrn2", mixer=dict(heads=width // 128, dim=128, vdim=128), mlp=moe)]
+    return dict(architecture="Kosalorn", vocab=65536, width=width, norm=dict(eps=1e-5), token_side=dict(dim=32),
+                layers=[dict(run[i % 4]) for i in range(layers)])
+
+
+def compare_workload(workload, sizes, dtype, steps, warmup, beside="lfm2"):
+    """Prefill and decode throughput of one design at some sizes, beside the closest model the engine has
+    (`beside`: LFM2 unless said) at equal layer sizes, through the same loops. `sizes`: (name, that model's
+    configuration, the design's)."""
     import torch
     from imparo_amd.engine.model import declared_tensors
     from imparo_amd.sampling import Sampler
     out = {"workload": workload, "dtype": dtype, "data": "synthetic token ids, random weights", "sizes": []}
     for name, lfm2, other in sizes:
         row = {"size": name}
-        for label, cfg in (("lfm2", lfm2), (workload, other)):
+        for label, cfg in ((beside, lfm2), (workload, other)):
             if cfg is None:
                 continue
             print(f"[bench] {name} {label}: writing random weights ...", file=sys.stderr, flush=True)
@@ -448,10 +472,10 @@ def compare_workload(workload, sizes, dtype, steps, warmup):
             row[label] = r
             del engine, sampler
             torch.cuda.empty_cache()
-        if "lfm2" in row and workload in row:
+        if beside in row and workload in row:
             for key in list(row[workload]):
                 if key.endswith("tok_s"):
-                    row.setdefault(f"{workload}_over_lfm2", {})[key] = round(row[workload][key] / row["lfm2"][key], 3)
+                    row.setdefault(f"{workload}_over_{beside}", {})[key] = round(row[workload][key] / row[beside][key], 3)
         out["sizes"].append(row)
     return out
 
@@ -475,6 +499,17 @@ def pupalorn_workload(dtype, steps, warmup, only=None, alone=False):
     return compare_workload("pupalorn", sizes, dtype, steps, warmup)
 
 
+def kosalorn_workload(dtype, steps, warmup, only=None, alone=False):
+    """The Kosalorn design at two sizes beside Pupalorn, the engine's closest model (attention in most layers over a
+    paged cache, a mixture of experts), at equal width, heads and depth. `only`: one size; `alone`: without Pupalorn."""
+    sizes = [
+        ("1.2B", pupalorn_shape(2048, 32, 8, 2048), kosalorn_shape(2048, 32, 1408, 5632)),
+        ("350M", pupalorn_shape(1024, 16, 8, 1152), kosalorn_shape(1024, 16, 768, 3072)),
+    ]
+    sizes = [(n, None if alone else a, b) for n, a, b in sizes if only in (None, n)]
+    return compare_workload("kosalorn", sizes, dtype, steps, warmup, beside="pupalorn")
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -486,14 +521,14 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64 and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="run only the 2,048-token prefill (for profiling)")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "long", "tumadra", "pupalorn"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "long", "tumadra", "pupalorn", "kosalorn"],
                     help="decode: the headline line (default). serving: continuous batching of 32 requests in 4 "
                          "waves (LFM2-700M shape). long: 64 requests of 32,768-token prompts, then 128 tokens "
                          "each (LFM2-350M shape). tumadra: prefill and decode of the Tumadra design at two sizes "
-                         "beside LFM2 at equal size; pupalorn: the same for the Pupalorn design. The last four "
-                         "print a line of their own")
-    ap.add_argument("--size", default=None, choices=["1.2B", "350M"], help="--workload pupalorn: one size only")
-    ap.add_argument("--alone", action="store_true", help="--workload pupalorn: without the LFM2 runs beside it")
+                         "beside LFM2 at equal size; pupalorn: the same for the Pupalorn design; kosalorn: the "
+                         "Kosalorn design beside Pupalorn. All but the first print a line of their own")
+    ap.add_argument("--size", default=None, choices=["1.2B", "350M"], help="--workload pupalorn or kosalorn: one size only")
+    ap.add_argument("--alone", action="store_true", help="--workload pupalorn or kosalorn: without the other model's runs beside it")
     ap.add_argument("--requests", type=int, default=64, help="--workload long: concurrent requests")
     ap.add_argument("--prompt-len", type=int, default=32768, help="--workload long: tokens per prompt")
     ap.add_argument("--portion", type=int, default=2048, help="--workload long: tokens of a prompt per step")
@@ -512,6 +547,9 @@ def main() -> int:
         return 0
     if args.workload == "pupalorn":
         print(json.dumps(pupalorn_workload(args.dtype, args.steps, args.warmup, args.size, args.alone)), flush=True)
+        return 0
+    if args.workload == "kosalorn":
+        print(json.dumps(kosalorn_workload(args.dtype, args.steps, args.warmup, args.size, args.alone)), flush=True)
         return 0
 
     import torch

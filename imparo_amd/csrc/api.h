@@ -148,9 +148,10 @@ int imparo_hgrn2_scan(const float* rows, int ld, int q_off, int f_off, int v_off
 
 // ---- pieces of a parallel block with gated sublayers
 // x += a * sigmoid(gates[:, :width]) (+ b * sigmoid(gates[:, width : 2 width]), b may be null); with `copy`
-// the new x is also stored there in copy_dtype. x, a, b float32 [tokens, width]; gates float32 [tokens, gate_ld].
-int imparo_gated_sum(float* x, const float* a, const float* b, const float* gates, int gate_ld, void* copy,
-                     int copy_dtype, int n_tokens, int width, imparo_stream stream);
+// the new x is also stored there in copy_dtype. x float32 [tokens, width]; a and b float32 [slices, tokens, width],
+// their slices added in order; gates float32 [tokens, gate_ld].
+int imparo_gated_sum(float* x, const float* a, int a_slices, const float* b, int b_slices, const float* gates,
+                     int gate_ld, void* copy, int copy_dtype, int n_tokens, int width, imparo_stream stream);
 // out[t, j] = gelu_tanh(z[t, j]) * table[ids[t], offset + j] for j < dim, zero for dim <= j < out_ld.
 int imparo_side_gate(const float* z, const void* table, int table_dtype, int table_ld, int offset, const int32_t* ids,
                      int vocab, void* out, int out_dtype, int n_tokens, int dim, int out_ld, imparo_stream stream);

@@ -14,33 +14,42 @@ __device__ __forceinline__ float gelu_tanh_f32(float z) {
     return 0.5f * z * (1.0f + tanhf(inner));
 }
 
-// gates [tokens, gate_ld]: columns 0 .. width are the first sublayer's, width .. 2 width the second's.
+// gates [tokens, gate_ld]: columns 0 .. width are the first sublayer's, width .. 2 width the second's. a and b
+// may come as sums over slices of a product's inner size, [slices, tokens, width], added here in order.
 template <typename TCopy>
-__global__ void k_gated_sum(float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ b,
-                            const float* __restrict__ gates, int gate_ld, TCopy* __restrict__ copy, int width,
-                            long long total) {
+__global__ void k_gated_sum(float* __restrict__ x, const float* __restrict__ a, int a_slices,
+                            const float* __restrict__ b, int b_slices, const float* __restrict__ gates, int gate_ld,
+                            TCopy* __restrict__ copy, int width, long long total) {
     const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= total) return;
     const long long t = i / width;
     const int c = (int)(i - t * width);
-    float sum = a[i] * sigmoid_f32(gates[t * gate_ld + c]);
-    if (b) sum += b[i] * sigmoid_f32(gates[t * gate_ld + width + c]);
+    float av = a[i];
+    for (int s = 1; s < a_slices; ++s) av += a[(long long)s * total + i];
+    float sum = av * sigmoid_f32(gates[t * gate_ld + c]);
+    if (b) {
+        float bv = b[i];
+        for (int s = 1; s < b_slices; ++s) bv += b[(long long)s * total + i];
+        sum += bv * sigmoid_f32(gates[t * gate_ld + width + c]);
+    }
     const float v = x[i] + sum;
     x[i] = v;
     if (copy) store_f32<TCopy>(copy, (size_t)i, v);
 }
 
-extern "C" int imparo_gated_sum(float* x, const float* a, const float* b, const float* gates, int gate_ld, void* copy,
-                                int copy_dtype, int n_tokens, int width, imparo_stream stream) {
+extern "C" int imparo_gated_sum(float* x, const float* a, int a_slices, const float* b, int b_slices,
+                                const float* gates, int gate_ld, void* copy, int copy_dtype, int n_tokens, int width,
+                                imparo_stream stream) {
     if (!x || !a || !gates || n_tokens < 0 || width < 1 || gate_ld < (b ? 2 * width : width)) return IMPARO_BAD_ARGUMENT;
+    if (a_slices < 1 || (b && b_slices < 1)) return IMPARO_BAD_ARGUMENT;
     if (n_tokens == 0) return IMPARO_OK;
     const long long total = (long long)n_tokens * width;
     const unsigned blocks = (unsigned)((total + 255) / 256);
     hipStream_t s = (hipStream_t)stream;
     if (copy && copy_dtype == IMPARO_BF16)
-        k_gated_sum<bf16_t><<<blocks, 256, 0, s>>>(x, a, b, gates, gate_ld, (bf16_t*)copy, width, total);
+        k_gated_sum<bf16_t><<<blocks, 256, 0, s>>>(x, a, a_slices, b, b_slices, gates, gate_ld, (bf16_t*)copy, width, total);
     else if (!copy || copy_dtype == IMPARO_F32)
-        k_gated_sum<float><<<blocks, 256, 0, s>>>(x, a, b, gates, gate_ld, (float*)copy, width, total);
+        k_gated_sum<float><<<blocks, 256, 0, s>>>(x, a, a_slices, b, b_slices, gates, gate_ld, (float*)copy, width, total);
     else
         return IMPARO_BAD_ARGUMENT;
     return launch_status();

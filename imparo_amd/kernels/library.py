@@ -76,7 +76,7 @@ _SIGNATURES = {
     "imparo_latent_store": [P, P, P, F, P, I, I, P, P, P, I, I, I, P, P, P, I, I, I, I, I, I, P],
     "imparo_head_gemm": [P, I, I, P, I, P, I, I, I, I, I, I, I, P],
     "imparo_hgrn2_scan": [P, I, I, I, I, P, P, P, P, P, P, I, I, I, I, P],
-    "imparo_gated_sum": [P, P, P, P, I, P, I, I, I, P],
+    "imparo_gated_sum": [P, P, I, P, I, P, I, P, I, I, I, P],
     "imparo_side_gate": [P, P, I, I, I, P, I, P, I, I, I, I, P],
     "imparo_add_rows": [P, P, c_int64, P],
     "imparo_moe_route_plan_tokens": [],

@@ -982,11 +982,14 @@ def hgrn2_scan(rows: torch.Tensor, q_off: int, f_off: int, v_off: int, lower: to
 # ---------------------------------------------------------------- a parallel block's elementwise pieces
 def gated_sum(x: torch.Tensor, a: torch.Tensor, b: Optional[torch.Tensor], gates: torch.Tensor,
               copy: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """x += a * sigmoid(gates[:, :width]) (+ b * sigmoid(gates[:, width:])); `copy` also receives the new x."""
+    """x += a * sigmoid(gates[:, :width]) (+ b * sigmoid(gates[:, width:])); `copy` also receives the new x.
+    a and b are shaped like x, or [slices, *x.shape]: sums over parts of a product's inner size, added in order."""
     n, width = x.shape
+    slices = lambda t: 1 if t is None or t.dim() == 2 else t.shape[0]
+    shaped = lambda t: (n, width) if t.dim() == 2 else (t.shape[0], n, width)
     _check(library().imparo_gated_sum(
-        _dev(x, "stream", torch.float32), _dev(a, "first sublayer's result", torch.float32, (n, width)),
-        _dev(b, "second sublayer's result", torch.float32, (n, width)),
+        _dev(x, "stream", torch.float32), _dev(a, "first sublayer's result", torch.float32, shaped(a)), slices(a),
+        _dev(b, "second sublayer's result", torch.float32, None if b is None else shaped(b)), slices(b),
         _dev(gates, "gates", torch.float32, (n, 2 * width if b is not None else gates.shape[1])), gates.shape[1],
         _dev(copy, "stream copy", None, (n, width)), _code(copy, "stream copy") if copy is not None else 0,
         n, width, _stream()), "gated_sum")

@@ -88,7 +88,7 @@ class Hgrn2:
                        ctx.seg_len, ctx.slot, o, H, dk, dv)
         normed = ctx.workspace.get("hgrn2_normed", (T, H * dv), self.out.in_dtype, alias="mixer_mid")
         ops.group_rms_norm(o, self.norm, H, self.eps, normed)
-        return self.out(ctx, normed, torch.float32, "mixer_out")
+        return self.out(ctx, normed, torch.float32, "mixer_out", sliced_ok=True)
 
 
 register_part("mixer", "hgrn2", Hgrn2)

@@ -135,7 +135,7 @@ class LatentAttention:
                              self.window)
         o = ws.get("latent_values", (T, H, self.vdim), self.out.in_dtype)
         ops.head_gemm(mixed.view(T, H, self.rank), self.w_values, o)
-        return self.out(ctx, o.view(T, H * self.vdim), torch.float32, "mixer_out")
+        return self.out(ctx, o.view(T, H * self.vdim), torch.float32, "mixer_out", sliced_ok=True)
 
 
 register_part("mixer", "latent_attention", LatentAttention)
