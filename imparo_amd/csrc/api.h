@@ -131,8 +131,22 @@ int imparo_attention_latent(const void* q, const void* rows_cache, void* out, in
 int imparo_latent_store(const float* q_rows, const float* kv_rows, const float* norm_weight, float eps,
                         const float* inv_freq, int n_freq, int interleaved, const int32_t* positions,
                         const int32_t* row_of_token, const int32_t* block_table, int table_stride, int page_size,
-                        int n_pages, void* cache, void* q_plain, void* q_full, int dtype, int n_tokens, int heads,
-                        int dim, int rot_dim, int rank, imparo_stream stream);
+                        int n_pages, void* cache, void* cache_t, void* q_plain, void* q_full, int dtype, int n_tokens,
+                        int heads, int dim, int rot_dim, int rank, imparo_stream stream);
+// (cache_t, or null: the normed latent once more at [pages, rank, page], for the matrix-core kernel below.)
+// The matrix-core form of imparo_attention_latent, bfloat16: up to 16 heads of a token are the 16 queries of a
+// wave's products. rows_t [pages, rank, page] holds the latents transposed inside a page; the values are the
+// latents (value_dim = rank). `_takes`: whether it is built for these sizes. `_split`: into how many parts the
+// keys are cut for this many tokens (and how many keys a part holds): with n_splits > 1, part_o [tokens, heads,
+// n_splits, rank] and part_ml [tokens, heads, n_splits, 2] float32 hold the parts, merged by a second launch.
+// `exact`: a softmax weight enters the product with the values as two bfloat16 numbers.
+int imparo_attention_latent_tiles_takes(int row_dim, int rank, int page_size);
+int imparo_attention_latent_tiles_split(int n_tokens, int heads, int max_context, int* split_keys);
+int imparo_attention_latent_tiles(const void* q, const void* rows, const void* rows_t, void* out, float* part_o,
+                                  float* part_ml, const int32_t* positions, const int32_t* row_of_token,
+                                  const int32_t* block_table, int table_stride, int page_size, int n_pages,
+                                  int n_tokens, int heads, int row_dim, int rank, float scale, int window,
+                                  int split_keys, int n_splits, int exact, imparo_stream stream);
 // out[t, h, :n] = W[h] in[t, h, :k] with w [heads, k, n]: a token's rows lie in_ld (out_ld) apart, a head's part
 // in_hs (out_hs) apart inside a row. float32 sums in the order of k.
 int imparo_head_gemm(const void* in, int in_ld, int in_hs, const void* w, int dtype, void* out, int out_dtype,

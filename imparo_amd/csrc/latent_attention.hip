@@ -37,7 +37,7 @@ __global__ __launch_bounds__(256) void k_latent_store(const float* __restrict__ 
                                                       const int32_t* __restrict__ row_of_token,
                                                       const int32_t* __restrict__ block_table, int table_stride,
                                                       int page_size, int n_pages, T* __restrict__ cache,
-                                                      T* __restrict__ q_plain, T* __restrict__ q_full, int heads, int dim,
+                                                      T* __restrict__ cache_t, T* __restrict__ q_plain, T* __restrict__ q_full, int heads, int dim,
                                                       int rot_dim, int rank) {
     __shared__ float sn[LAT_MAX_FREQ], cs[LAT_MAX_FREQ];
     __shared__ float scratch[16];
@@ -56,6 +56,11 @@ __global__ __launch_bounds__(256) void k_latent_store(const float* __restrict__ 
             for (int i = threadIdx.x; i < rank; i += blockDim.x) store_f32<T>(dst, i, kv[i] * scale * norm_weight[i]);
             for (int d = threadIdx.x; d < rot_dim; d += blockDim.x)
                 store_f32<T>(dst, rank + d, turned(kv + rank, d, n_freq, interleaved, sn, cs));
+            if (cache_t) {      // the latent once more, [page, rank, position]: the values as the matrix-core kernel reads them
+                T* dst_t = cache_t + (size_t)page * rank * page_size + (pos % page_size);
+                for (int i = threadIdx.x; i < rank; i += blockDim.x)
+                    store_f32<T>(dst_t, (size_t)i * page_size, kv[i] * scale * norm_weight[i]);
+            }
         }
     }
     const int per = dim + rot_dim;
@@ -73,23 +78,24 @@ __global__ __launch_bounds__(256) void k_latent_store(const float* __restrict__ 
 extern "C" int imparo_latent_store(const float* q_rows, const float* kv_rows, const float* norm_weight, float eps,
                                    const float* inv_freq, int n_freq, int interleaved, const int32_t* positions,
                                    const int32_t* row_of_token, const int32_t* block_table, int table_stride,
-                                   int page_size, int n_pages, void* cache, void* q_plain, void* q_full, int dtype,
+                                   int page_size, int n_pages, void* cache, void* cache_t, void* q_plain, void* q_full, int dtype,
                                    int n_tokens, int heads, int dim, int rot_dim, int rank, imparo_stream stream) {
     if (!q_rows || !kv_rows || !norm_weight || !positions || !q_plain || !q_full) return IMPARO_BAD_ARGUMENT;
     if (n_tokens < 0 || heads < 1 || dim < 1 || rot_dim < 0 || rank < 1) return IMPARO_BAD_ARGUMENT;
     if (n_freq < 0 || n_freq > LAT_MAX_FREQ || 2 * n_freq > rot_dim || (n_freq && !inv_freq)) return IMPARO_BAD_ARGUMENT;
+    if (cache_t && !cache) return IMPARO_BAD_ARGUMENT;
     if (cache && (!row_of_token || !block_table || table_stride < 1 || page_size < 1 || n_pages < 1)) return IMPARO_BAD_ARGUMENT;
     if (n_tokens == 0) return IMPARO_OK;
     hipStream_t s = (hipStream_t)stream;
     if (dtype == IMPARO_F32)
         k_latent_store<float><<<n_tokens, 256, 0, s>>>(q_rows, kv_rows, norm_weight, eps, inv_freq, n_freq, interleaved,
                                                        positions, row_of_token, block_table, table_stride, page_size,
-                                                       n_pages, (float*)cache, (float*)q_plain, (float*)q_full, heads, dim,
+                                                       n_pages, (float*)cache, (float*)cache_t, (float*)q_plain, (float*)q_full, heads, dim,
                                                        rot_dim, rank);
     else if (dtype == IMPARO_BF16)
         k_latent_store<bf16_t><<<n_tokens, 256, 0, s>>>(q_rows, kv_rows, norm_weight, eps, inv_freq, n_freq, interleaved,
                                                         positions, row_of_token, block_table, table_stride, page_size,
-                                                        n_pages, (bf16_t*)cache, (bf16_t*)q_plain, (bf16_t*)q_full, heads,
+                                                        n_pages, (bf16_t*)cache, (bf16_t*)cache_t, (bf16_t*)q_plain, (bf16_t*)q_full, heads,
                                                         dim, rot_dim, rank);
     else
         return IMPARO_BAD_ARGUMENT;
@@ -151,6 +157,285 @@ extern "C" int imparo_head_gemm(const void* in, int in_ld, int in_hs, const void
                                                           out_ld, out_hs, n_tokens, k, n);
     else
         return IMPARO_BAD_ARGUMENT;
+    return launch_status();
+}
+
+// ---------------------------------------------------------------- the matrix-core kernel
+// A wave takes up to 16 heads of one token as the 16 queries of its products: every head reads the same
+// rows, so one tile of keys serves them all, and they share one range of keys. Keys are walked in tiles of
+// 32 at absolute multiples of 32:
+//   S^T[key][head] = rows . Q^T     A = 16 bytes of a cached row a lane, B = Q^T in registers. Row m of
+//                                   product t stands for key 8 (m / 4) + 4 t + m % 4, so that the 8 scores
+//                                   a lane ends up with are the keys 8 (lane / 16) .. + 7,
+//   O^T[dim][head] += V^T . P^T     A = 16 bytes of the transposed copy of the latents (8 keys of one
+//                                   dimension), B = the lane's 8 softmax weights as they are.
+// With `exact` a weight enters the second product as two bfloat16 numbers (its rounding and what the
+// rounding lost). With n_splits > 1 a wave takes the keys [split * split_keys, (split + 1) * split_keys)
+// of its range and writes an unnormed part (sum, maximum, weight sum); k_latent_merge adds the parts.
+typedef float lat_f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 lat_bf16x8 __attribute__((ext_vector_type(8)));
+union LatFrag {
+    uint4 u;
+    lat_bf16x8 v;
+};
+
+#define LAT_WAVES 4
+
+__device__ __forceinline__ uint32_t lat_pack2(float a, float b) {
+    return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+}
+
+__device__ __forceinline__ float lat_bf16_value(float a) { return __uint_as_float((uint32_t)f32_to_bf16(a) << 16); }
+
+template <int NK, int NV>
+__global__ __launch_bounds__(LAT_WAVES * WAVE) void k_latent_attention_tiles(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ rows, const bf16_t* __restrict__ rows_t,
+    bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ row_of_token,
+    const int32_t* __restrict__ block_table, int table_stride, int page_shift, int n_pages, int n_tokens, int heads,
+    int row_dim, int rank, float scale, int window, int split_keys, int n_splits, int exact) {
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+    const int c = lane & 15, g = lane >> 4;
+    const int head_groups = (heads + 15) / 16;
+    const long long total = (long long)n_tokens * head_groups * n_splits;
+    const long long id = (long long)blockIdx.x * LAT_WAVES + wave;
+    if (id >= total) return;                       // (no barrier below: waves are on their own)
+    const int split = (int)(id % n_splits);
+    const long long rest = id / n_splits;
+    const int t = (int)(rest % n_tokens);
+    const int h = (int)(rest / n_tokens) * 16 + c;  // this lane's head
+    const bool live = h < heads;
+    const int pos = positions[t];
+    const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
+    const int k_lo = n_splits > 1 ? max(lo, split * split_keys) : lo;
+    const int k_hi = n_splits > 1 ? min(pos, (split + 1) * split_keys - 1) : pos;
+    const int page_size = 1 << page_shift, page_mask = page_size - 1;
+    const int32_t* table = block_table + (size_t)row_of_token[t] * table_stride;
+
+    LatFrag qf[NK];
+    {
+        const bf16_t* qrow = q + ((size_t)t * heads + (live ? h : 0)) * row_dim;
+#pragma unroll
+        for (int dk = 0; dk < NK; ++dk) {
+            const int d0 = dk * 32 + 8 * g;
+            qf[dk].u = (live && d0 < row_dim) ? *reinterpret_cast<const uint4*>(qrow + d0) : make_uint4(0u, 0u, 0u, 0u);
+        }
+    }
+    lat_f32x4 o[NV];
+#pragma unroll
+    for (int dt = 0; dt < NV; ++dt) o[dt] = lat_f32x4{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+
+    if (k_lo <= k_hi) {
+        for (int base = k_lo & ~31; base <= k_hi; base += 32) {
+            LatFrag kf[2][NK];
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2) {
+                const int key = min(max(base + 8 * (c >> 2) + 4 * t2 + (c & 3), k_lo), k_hi);
+                const int page = min(max(table[key >> page_shift], 0), n_pages - 1);
+                const bf16_t* krow = rows + ((size_t)page * page_size + (key & page_mask)) * row_dim;
+#pragma unroll
+                for (int dk = 0; dk < NK; ++dk)     // beyond the row: its last 8 again, against zeros of the query
+                    kf[t2][dk].u = *reinterpret_cast<const uint4*>(krow + min(dk * 32 + 8 * g, row_dim - 8));
+            }
+            const int kg = base + 8 * g;            // this lane's 8 keys in both products' results
+            LatFrag vf[NV];
+            {
+                const int kgc = min(max(kg, k_lo & ~7), k_hi & ~7);
+                const int page = min(max(table[kgc >> page_shift], 0), n_pages - 1);
+                const bf16_t* vbase = rows_t + (size_t)page * rank * page_size + (kgc & page_mask);
+#pragma unroll
+                for (int dt = 0; dt < NV; ++dt)
+                    vf[dt].u = *reinterpret_cast<const uint4*>(vbase + (size_t)min(dt * 16 + c, rank - 1) * page_size);
+            }
+            lat_f32x4 s[2];
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2) {
+                s[t2] = lat_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int dk = 0; dk < NK; ++dk)
+                    s[t2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t2][dk].v, qf[dk].v, s[t2], 0, 0, 0);
+            }
+            float sv[8];
+            float tile_max = -INFINITY;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int key = kg + j;
+                sv[j] = (key >= k_lo && key <= k_hi) ? s[j >> 2][j & 3] * scale : -INFINITY;
+                tile_max = fmaxf(tile_max, sv[j]);
+            }
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE));
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE));
+            const float m_new = fmaxf(m, tile_max);  // finite: every tile holds a key of the range
+            const float corr = expf(m - m_new);
+            float p[8], p_sum = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                p[j] = expf(sv[j] - m_new);
+                p_sum += p[j];
+            }
+            l = l * corr + p_sum;                   // a lane's own 8 keys; the four lanes of a head are added at the end
+            m = m_new;
+#pragma unroll
+            for (int dt = 0; dt < NV; ++dt) o[dt] *= corr;
+            if (base < k_lo || base + 31 > k_hi) {  // what a page holds beyond the range may be anything: zeros instead
+                uint32_t keep[4];
+#pragma unroll
+                for (int j2 = 0; j2 < 4; ++j2) {
+                    const int k0 = kg + 2 * j2;
+                    keep[j2] = ((k0 >= k_lo && k0 <= k_hi) ? 0x0000ffffu : 0u) |
+                               ((k0 + 1 >= k_lo && k0 + 1 <= k_hi) ? 0xffff0000u : 0u);
+                }
+#pragma unroll
+                for (int dt = 0; dt < NV; ++dt)
+                    vf[dt].u = make_uint4(vf[dt].u.x & keep[0], vf[dt].u.y & keep[1], vf[dt].u.z & keep[2], vf[dt].u.w & keep[3]);
+            }
+            LatFrag ph;
+            ph.u = make_uint4(lat_pack2(p[0], p[1]), lat_pack2(p[2], p[3]), lat_pack2(p[4], p[5]), lat_pack2(p[6], p[7]));
+#pragma unroll
+            for (int dt = 0; dt < NV; ++dt)
+                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, ph.v, o[dt], 0, 0, 0);
+            if (exact) {
+                float r[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) r[j] = p[j] - lat_bf16_value(p[j]);
+                LatFrag pl;
+                pl.u = make_uint4(lat_pack2(r[0], r[1]), lat_pack2(r[2], r[3]), lat_pack2(r[4], r[5]), lat_pack2(r[6], r[7]));
+#pragma unroll
+                for (int dt = 0; dt < NV; ++dt)
+                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pl.v, o[dt], 0, 0, 0);
+            }
+        }
+    }
+    l += __shfl_xor(l, 16, WAVE);
+    l += __shfl_xor(l, 32, WAVE);
+    if (!live) return;
+    const size_t row = (size_t)t * heads + h;
+    if (n_splits == 1) {
+        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        bf16_t* dst = out + row * rank;
+#pragma unroll
+        for (int dt = 0; dt < NV; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int d = dt * 16 + 4 * g + i;
+                if (d < rank) dst[d] = f32_to_bf16(o[dt][i] * inv);
+            }
+    } else {
+        float* dst = part_o + (row * n_splits + split) * rank;
+#pragma unroll
+        for (int dt = 0; dt < NV; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int d = dt * 16 + 4 * g + i;
+                if (d < rank) dst[d] = o[dt][i];
+            }
+        if (g == 0) {
+            part_ml[(row * n_splits + split) * 2] = m;
+            part_ml[(row * n_splits + split) * 2 + 1] = l;
+        }
+    }
+}
+
+// out[row, d] = sum_s w_s part_o[row, s, d] / sum_s w_s l_s with w_s = exp(m_s - max m), the parts in order.
+__global__ void k_latent_merge(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                               bf16_t* __restrict__ out, long long n_rows, int n_splits, int rank) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_rows * rank) return;
+    const long long row = i / rank;
+    const int d = (int)(i - row * rank);
+    const float* ml = part_ml + row * n_splits * 2;
+    float top = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) top = fmaxf(top, ml[2 * s]);
+    float num = 0.f, den = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+        const float ms = ml[2 * s];
+        if (ms == -INFINITY) continue;
+        const float w = expf(ms - top);
+        num += w * part_o[(row * n_splits + s) * rank + d];
+        den += w * ml[2 * s + 1];
+    }
+    out[i] = f32_to_bf16(den > 0.f ? num / den : 0.f);
+}
+
+// The sizes the matrix-core kernel is built for: latents of up to 256 numbers in steps of 8 (value tiles of
+// 16: 2, 4, 8 or 16 of them), rows (latent and rotated key part) of up to 32 (tiles / 2 + 2) numbers in
+// steps of 8, pages of a power of two from 32 on.
+static int latent_tiles_shape(int row_dim, int rank, int* nk, int* nv) {
+    if (rank < 8 || rank > 256 || rank % 8 || row_dim % 8 || row_dim < rank) return 0;
+    const int v = rank <= 32 ? 2 : rank <= 64 ? 4 : rank <= 128 ? 8 : 16;
+    const int k = (row_dim + 31) / 32;
+    if (k > v / 2 + 2) return 0;
+    *nv = v;
+    *nk = k <= v / 2 + 1 ? v / 2 + 1 : v / 2 + 2;
+    return 1;
+}
+
+extern "C" int imparo_attention_latent_tiles_takes(int row_dim, int rank, int page_size) {
+    int nk, nv;
+    return page_size >= 32 && (page_size & (page_size - 1)) == 0 && latent_tiles_shape(row_dim, rank, &nk, &nv);
+}
+
+// Into how many parts the keys of a launch are cut, and how many keys a part holds: few tokens over long
+// contexts would leave most of the chip idle. Parts lie at absolute multiples of their size.
+extern "C" int imparo_attention_latent_tiles_split(int n_tokens, int heads, int max_context, int* split_keys) {
+    const long long items = (long long)n_tokens * ((heads + 15) / 16);
+    int want = items >= 512 ? 1 : (int)((512 + items - 1) / items);
+    int keys = ((max_context + want - 1) / want + 63) / 64 * 64;
+    if (keys < 64) keys = 64;
+    const int n = max_context <= keys ? 1 : (max_context + keys - 1) / keys;
+    if (split_keys) *split_keys = keys;
+    return n;
+}
+
+template <int NK, int NV>
+static void launch_latent_tiles(const void* q, const void* rows, const void* rows_t, void* out, float* part_o,
+                                float* part_ml, const int32_t* positions, const int32_t* row_of_token,
+                                const int32_t* block_table, int table_stride, int page_shift, int n_pages, int n_tokens,
+                                int heads, int row_dim, int rank, float scale, int window, int split_keys, int n_splits,
+                                int exact, hipStream_t s) {
+    const long long waves = (long long)n_tokens * ((heads + 15) / 16) * n_splits;
+    const unsigned blocks = (unsigned)((waves + LAT_WAVES - 1) / LAT_WAVES);
+    k_latent_attention_tiles<NK, NV><<<blocks, LAT_WAVES * WAVE, 0, s>>>(
+        (const bf16_t*)q, (const bf16_t*)rows, (const bf16_t*)rows_t, (bf16_t*)out, part_o, part_ml, positions,
+        row_of_token, block_table, table_stride, page_shift, n_pages, n_tokens, heads, row_dim, rank, scale, window,
+        split_keys, n_splits, exact);
+}
+
+// q [tokens, heads, row_dim], rows [pages, page, row_dim], rows_t [pages, rank, page] (the latents once more,
+// transposed inside a page), out [tokens, heads * rank], all bfloat16. n_splits and split_keys as
+// imparo_attention_latent_tiles_split gives them for a max_context that bounds every position + 1; with
+// n_splits > 1, part_o [tokens, heads, n_splits, rank] and part_ml [tokens, heads, n_splits, 2] float32.
+extern "C" int imparo_attention_latent_tiles(const void* q, const void* rows, const void* rows_t, void* out,
+                                             float* part_o, float* part_ml, const int32_t* positions,
+                                             const int32_t* row_of_token, const int32_t* block_table, int table_stride,
+                                             int page_size, int n_pages, int n_tokens, int heads, int row_dim, int rank,
+                                             float scale, int window, int split_keys, int n_splits, int exact,
+                                             imparo_stream stream) {
+    if (!q || !rows || !rows_t || !out || !positions || !row_of_token || !block_table) return IMPARO_BAD_ARGUMENT;
+    if (n_tokens < 0 || heads < 1 || table_stride < 1 || n_pages < 1 || window < 0) return IMPARO_BAD_ARGUMENT;
+    int nk = 0, nv = 0;
+    if (!imparo_attention_latent_tiles_takes(row_dim, rank, page_size) || !latent_tiles_shape(row_dim, rank, &nk, &nv))
+        return IMPARO_BAD_ARGUMENT;
+    if (n_splits < 1 || (n_splits > 1 && (!part_o || !part_ml || split_keys < 32 || split_keys % 32))) return IMPARO_BAD_ARGUMENT;
+    if (n_splits > 1 && (long long)n_splits * split_keys > 0x7fffffffLL) return IMPARO_BAD_ARGUMENT;
+    if (n_tokens == 0) return IMPARO_OK;
+    int page_shift = 0;
+    while ((1 << page_shift) < page_size) ++page_shift;
+    hipStream_t s = (hipStream_t)stream;
+#define LAT_CASE(K, V)                                                                                               \
+    if (nk == K && nv == V)                                                                                          \
+        launch_latent_tiles<K, V>(q, rows, rows_t, out, part_o, part_ml, positions, row_of_token, block_table,       \
+                                  table_stride, page_shift, n_pages, n_tokens, heads, row_dim, rank, scale, window,  \
+                                  split_keys, n_splits, exact, s);
+    LAT_CASE(2, 2) LAT_CASE(3, 2) LAT_CASE(3, 4) LAT_CASE(4, 4) LAT_CASE(5, 8) LAT_CASE(6, 8) LAT_CASE(9, 16) LAT_CASE(10, 16)
+#undef LAT_CASE
+    if (launch_status() != IMPARO_OK) return IMPARO_LAUNCH_FAILED;
+    if (n_splits > 1) {
+        const long long n = (long long)n_tokens * heads * rank;
+        k_latent_merge<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, (long long)n_tokens * heads,
+                                                                  n_splits, rank);
+    }
     return launch_status();
 }
 

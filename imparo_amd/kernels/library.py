@@ -73,7 +73,10 @@ _SIGNATURES = {
     "imparo_moe_route": [P, P, P, P, I, I, I, I, P],
     "imparo_moe_gated": [P, P, P, P, I, I, I, P],
     "imparo_attention_latent": [P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P],
-    "imparo_latent_store": [P, P, P, F, P, I, I, P, P, P, I, I, I, P, P, P, I, I, I, I, I, I, P],
+    "imparo_latent_store": [P, P, P, F, P, I, I, P, P, P, I, I, I, P, P, P, P, I, I, I, I, I, I, P],
+    "imparo_attention_latent_tiles_takes": [I, I, I],
+    "imparo_attention_latent_tiles_split": [I, I, I, P],
+    "imparo_attention_latent_tiles": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, I, I, P],
     "imparo_head_gemm": [P, I, I, P, I, P, I, I, I, I, I, I, I, P],
     "imparo_hgrn2_scan": [P, I, I, I, I, P, P, P, P, P, P, I, I, I, I, P],
     "imparo_gated_sum": [P, P, I, P, I, P, I, P, I, I, I, P],

@@ -9,6 +9,8 @@ from __future__ import annotations
 
 from typing import Optional
 
+import ctypes
+
 import torch
 
 from .library import library
@@ -904,9 +906,11 @@ def post_norm_add(x: torch.Tensor, delta, w_post: torch.Tensor, eps_post: float,
 def latent_store(q_rows: torch.Tensor, kv_rows: torch.Tensor, norm_weight: torch.Tensor, eps: float,
                  inv_freq: Optional[torch.Tensor], interleaved: bool, positions: torch.Tensor, row_of_token: torch.Tensor,
                  block_table: Optional[torch.Tensor], page_size: int, cache: Optional[torch.Tensor], q_plain: torch.Tensor,
-                 q_full: torch.Tensor, heads: int, dim: int, rot_dim: int, rank: int) -> None:
+                 q_full: torch.Tensor, heads: int, dim: int, rot_dim: int, rank: int,
+                 cache_t: Optional[torch.Tensor] = None) -> None:
     """The latent's norm, the rotation of the shared key part and of every head's rotated query part, the write
-    of [latent | rotated key part] into the token's page, and the queries laid out for the absorbed products."""
+    of [latent | rotated key part] into the token's page, and the queries laid out for the absorbed products.
+    `cache_t` [pages, rank, page]: the latent is written there once more, transposed inside the page."""
     n = q_rows.shape[0]
     n_freq = 0 if inv_freq is None else inv_freq.shape[0]
     n_pages = table_stride = 0
@@ -916,6 +920,10 @@ def latent_store(q_rows: torch.Tensor, kv_rows: torch.Tensor, norm_weight: torch
         if block_table is None or block_table.dim() != 2:
             raise KernelArgumentError("latent_store: a [rows, pages] block table is needed to write the cache")
         table_stride = block_table.shape[1]
+        if cache_t is not None:
+            _dev(cache_t, "transposed latents", q_full.dtype, (n_pages, rank, page_size))
+    elif cache_t is not None:
+        raise KernelArgumentError("latent_store: the transposed latents are written with the rows only")
     _check(library().imparo_latent_store(
         _dev(q_rows, "query rows", torch.float32, (n, heads * (dim + rot_dim))),
         _dev(kv_rows, "latent rows", torch.float32, (n, rank + rot_dim)),
@@ -923,7 +931,7 @@ def latent_store(q_rows: torch.Tensor, kv_rows: torch.Tensor, norm_weight: torch
         _dev(inv_freq, "inverse frequencies", torch.float32), n_freq, int(interleaved),
         _dev(positions, "positions", torch.int32, (n,)), _dev(row_of_token, "row_of_token", torch.int32, (n,)),
         _dev(block_table, "block table", torch.int32), table_stride, page_size, n_pages, _dev(cache, "latent cache"),
-        _dev(q_plain, "unrotated queries", q_full.dtype, (n, heads, dim)),
+        _dev(cache_t, "transposed latents"), _dev(q_plain, "unrotated queries", q_full.dtype, (n, heads, dim)),
         _dev(q_full, "queries", None, (n, heads, rank + rot_dim)), _code(q_full, "queries"),
         n, heads, dim, rot_dim, rank, _stream()), "latent_store")
 
@@ -958,6 +966,54 @@ def attention_latent(q: torch.Tensor, cache: torch.Tensor, out: torch.Tensor, po
         _code(q, "q"), _dev(positions, "positions", torch.int32, (n,)), _dev(row_of_token, "row_of_token", torch.int32, (n,)),
         _dev(block_table, "block table", torch.int32), block_table.shape[1], page_size, n, heads, row_dim, value_dim,
         n_pages, float(scale), int(window or 0), _stream()), "attention_latent")
+    return out
+
+
+def attention_latent_tiles_takes(dtype: torch.dtype, row_dim: int, rank: int, page_size: int) -> bool:
+    """Whether the matrix-core kernel over cached latents is built for these sizes."""
+    if dtype != torch.bfloat16 or page_size < 32 or page_size & (page_size - 1):
+        return False
+    if rank < 8 or rank > 256 or rank % 8 or row_dim % 8 or row_dim < rank:
+        return False
+    value_tiles = 2 if rank <= 32 else 4 if rank <= 64 else 8 if rank <= 128 else 16
+    return (row_dim + 31) // 32 <= value_tiles // 2 + 2
+
+
+def attention_latent_tiles_split(n_tokens: int, heads: int, max_context: int):
+    """(parts the keys of such a launch are cut into, keys a part)."""
+    keys = ctypes.c_int(0)
+    n = int(library().imparo_attention_latent_tiles_split(int(n_tokens), int(heads), int(max_context), ctypes.byref(keys)))
+    return n, int(keys.value)
+
+
+def attention_latent_tiles(q: torch.Tensor, cache: torch.Tensor, cache_t: torch.Tensor, out: torch.Tensor,
+                           positions: torch.Tensor, row_of_token: torch.Tensor, block_table: torch.Tensor, scale: float,
+                           window: Optional[int], n_splits: int = 1, split_keys: int = 0,
+                           part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None,
+                           exact: bool = True) -> torch.Tensor:
+    """attention_latent on the matrix cores (bfloat16): up to 16 heads of a token share a wave and every tile
+    of keys. `cache_t` [pages, rank, page] holds the latents transposed inside a page; the values are the
+    latents. `n_splits`, `split_keys` from attention_latent_tiles_split for a context bound that holds for every
+    token; with n_splits > 1 `part_o` (tokens * heads * n_splits * rank) and `part_ml` (tokens * heads * n_splits
+    * 2) float32 hold the parts. `exact`: the softmax weights keep float32's precision through the second product."""
+    n, heads, row_dim = q.shape
+    n_pages, page_size, rd = cache.shape
+    rank = cache_t.shape[1]
+    if rd != row_dim or not attention_latent_tiles_takes(q.dtype, row_dim, rank, page_size):
+        raise KernelArgumentError(f"attention_latent_tiles: rows of {row_dim} (cache {rd}), latents of {rank}, pages of "
+                                  f"{page_size}, {q.dtype} are not taken")
+    if n_splits > 1:
+        if part_o is None or part_ml is None or part_o.numel() < n * heads * n_splits * rank or part_ml.numel() < n * heads * n_splits * 2:
+            raise KernelArgumentError("attention_latent_tiles: the buffers for the parts are missing or too small")
+    _check(library().imparo_attention_latent_tiles(
+        _dev(q, "q", torch.bfloat16), _dev(cache, "latent cache", torch.bfloat16),
+        _dev(cache_t, "transposed latents", torch.bfloat16, (n_pages, rank, page_size)),
+        _dev(out, "attention out", torch.bfloat16, (n, heads * rank)),
+        _dev(part_o, "part_o", torch.float32) if n_splits > 1 else None,
+        _dev(part_ml, "part_ml", torch.float32) if n_splits > 1 else None,
+        _dev(positions, "positions", torch.int32, (n,)), _dev(row_of_token, "row_of_token", torch.int32, (n,)),
+        _dev(block_table, "block table", torch.int32), block_table.shape[1], page_size, n_pages, n, heads, row_dim, rank,
+        float(scale), int(window or 0), int(split_keys), int(n_splits), int(bool(exact)), _stream()), "attention_latent_tiles")
     return out
 
 

@@ -79,6 +79,7 @@ class LatentAttention:
         self.window: Optional[int] = spec.get("window")
         self.eps = float(spec["eps"])
         self.row_dim = self.rank + self.rot_dim
+        self.tiles = False        # whether the matrix-core kernel runs (cache_spec decides, with the page size)
         if self.row_dim > ops.ATTENTION_MAX_HEAD_DIM:
             raise ValueError(f"a cached row of {self.row_dim} numbers (kv_rank + rot_dim) passes the attention "
                              f"kernel's {ops.ATTENTION_MAX_HEAD_DIM}")
@@ -108,7 +109,13 @@ class LatentAttention:
 
     def cache_spec(self, page_size: int) -> PagedSpec:
         """One row [latent | rotated key part] a position, shared by all heads."""
-        return PagedSpec((PagedArray("latent", (PAGE, self.row_dim)),), self.window)
+        self.tiles = ops.attention_latent_tiles_takes(self.engine_dtype, self.row_dim, self.rank, page_size)
+        arrays = (PagedArray("latent", (PAGE, self.row_dim)),)
+        if self.tiles:
+            # the latents once more, transposed inside a page: the matrix-core kernel's second product reads
+            # 8 positions of one number of the latent in one load
+            arrays += (PagedArray("latent_t", (self.rank, PAGE)),)
+        return PagedSpec(arrays, self.window)
 
     def forward(self, ctx: StepContext, site: int, owns_cache: bool, h: torch.Tensor) -> torch.Tensor:
         T, H = h.shape[0], self.heads
@@ -128,11 +135,21 @@ class LatentAttention:
         ops.latent_store(q_rows, kv_rows, self.kv_norm, self.eps, self.position.inv_freq,
                          bool(getattr(self.position, "interleaved", False)), ctx.positions, ctx.row_of_token,
                          table if owns_cache else None, ctx.page_size, cache if owns_cache else None,
-                         q_plain, q_full, H, self.dim, self.rot_dim, self.rank)
+                         q_plain, q_full, H, self.dim, self.rot_dim, self.rank,
+                         cache_t=arrays["latent_t"] if self.tiles and owns_cache else None)
         ops.head_gemm(q_plain, self.w_absorb, q_full)               # columns 0 .. rank of every head's query
         mixed = ws.get("latent_mixed", (T, H * self.rank), ctx.dtype, alias="mixer_mid")
-        ops.attention_latent(q_full, cache, mixed, ctx.positions, ctx.row_of_token, table, self.rank, self.scale,
-                             self.window)
+        if self.tiles:
+            n_splits, split_keys = ops.attention_latent_tiles_split(T, H, ctx.max_context)
+            part_o = part_ml = None
+            if n_splits > 1:
+                part_o = ws.get("latent_part_o", (T * H * n_splits * self.rank,), torch.float32)
+                part_ml = ws.get("latent_part_ml", (T * H * n_splits * 2,), torch.float32)
+            ops.attention_latent_tiles(q_full, cache, arrays["latent_t"], mixed, ctx.positions, ctx.row_of_token, table,
+                                       self.scale, self.window, n_splits, split_keys, part_o, part_ml)
+        else:
+            ops.attention_latent(q_full, cache, mixed, ctx.positions, ctx.row_of_token, table, self.rank, self.scale,
+                                 self.window)
         o = ws.get("latent_values", (T, H, self.vdim), self.out.in_dtype)
         ops.head_gemm(mixed.view(T, H, self.rank), self.w_values, o)
         return self.out(ctx, o.view(T, H * self.vdim), torch.float32, "mixer_out", sliced_ok=True)
