@@ -152,13 +152,23 @@ int imparo_attention_latent_tiles(const void* q, const void* rows, const void* r
 int imparo_head_gemm(const void* in, int in_ld, int in_hs, const void* w, int dtype, void* out, int out_dtype,
                      int out_ld, int out_hs, int n_tokens, int heads, int k, int n, imparo_stream stream);
 
+// The same product on the matrix cores: in bfloat16, w_t [heads, n, k] (the inner size running fastest) bfloat16,
+// out bfloat16 or float32; k, in_ld and in_hs multiples of 8.
+int imparo_head_gemm_tiles(const void* in, int in_ld, int in_hs, const void* w_t, void* out, int out_dtype, int out_ld,
+                           int out_hs, int n_tokens, int heads, int k, int n, imparo_stream stream);
+
 // ---- a gated linear recurrence with a matrix of state a head
 // Per request (row), head and token in order: q = silu(zq), f = lower + (1 - lower) sigmoid(zf),
 // S <- diag(f) S + (1 - f) v^T, out = S^T q. rows [tokens, ld] float32 holds zq at q_off, zf at f_off, v at v_off,
 // head by head; state [slots, heads, dim, vdim] float32; out [tokens, heads * vdim] float32. dim <= 256.
+// chunk_tokens 0: one launch, a block walks a row's whole segment. Otherwise (a multiple of 8) segments are walked
+// in chunks of that many tokens side by side, in three launches; max_chunks >= ceil(longest segment /
+// chunk_tokens); chunk_state [n_rows * max_chunks, heads, dim, vdim] and chunk_decay [n_rows * max_chunks, heads,
+// dim] float32 are scratch.
 int imparo_hgrn2_scan(const float* rows, int ld, int q_off, int f_off, int v_off, const float* lower, float* state,
                       const int32_t* seg_start, const int32_t* seg_len, const int32_t* slot, float* out, int n_rows,
-                      int heads, int dim, int vdim, imparo_stream stream);
+                      int heads, int dim, int vdim, int chunk_tokens, int max_chunks, float* chunk_state,
+                      float* chunk_decay, imparo_stream stream);
 
 // ---- pieces of a parallel block with gated sublayers
 // x += a * sigmoid(gates[:, :width]) (+ b * sigmoid(gates[:, width : 2 width]), b may be null); with `copy`

@@ -439,6 +439,64 @@ extern "C" int imparo_attention_latent_tiles(const void* q, const void* rows, co
     return launch_status();
 }
 
+// The per-head product on the matrix cores, bfloat16: w_t [heads, n, k] keeps a head's matrix with the inner
+// size running fastest, as both operands of a 16x16x32 product want it. A wave makes 16 outputs of one head
+// for 16 tokens: O^T[n][token] = W_t . in^T, so that a lane ends up with 4 neighbouring outputs of one token.
+template <typename TOut>
+__global__ __launch_bounds__(LAT_WAVES * WAVE) void k_head_gemm_tiles(const bf16_t* __restrict__ in, int in_ld, int in_hs,
+                                                                      const bf16_t* __restrict__ w_t, TOut* __restrict__ out,
+                                                                      int out_ld, int out_hs, int n_tokens, int K, int N) {
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+    const int c = lane & 15, g = lane >> 4;
+    const int h = blockIdx.y;
+    const int n_base = (blockIdx.z * LAT_WAVES + wave) * 16;
+    if (n_base >= N) return;
+    const int token = blockIdx.x * 16 + c;
+    const bool live = token < n_tokens;
+    const bf16_t* arow = w_t + ((size_t)h * N + min(n_base + c, N - 1)) * K;
+    const bf16_t* brow = in + (size_t)(live ? token : 0) * in_ld + (size_t)h * in_hs;
+    lat_f32x4 acc = lat_f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < K; k0 += 32) {
+        const int kk = k0 + 8 * g;
+        LatFrag a, b;
+        a.u = kk < K ? *reinterpret_cast<const uint4*>(arow + kk) : make_uint4(0u, 0u, 0u, 0u);
+        b.u = (kk < K && live) ? *reinterpret_cast<const uint4*>(brow + kk) : make_uint4(0u, 0u, 0u, 0u);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc, 0, 0, 0);
+    }
+    if (!live) return;
+    TOut* dst = out + (size_t)token * out_ld + (size_t)h * out_hs;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int n = n_base + 4 * g + i;
+        if (n < N) store_f32<TOut>(dst, n, acc[i]);
+    }
+}
+
+// in [tokens, .] bfloat16 (a token's rows in_ld apart, a head's part in_hs apart, both multiples of 8, as is k),
+// w_t [heads, n, k] bfloat16, out bfloat16 or float32.
+extern "C" int imparo_head_gemm_tiles(const void* in, int in_ld, int in_hs, const void* w_t, void* out, int out_dtype,
+                                      int out_ld, int out_hs, int n_tokens, int heads, int k, int n,
+                                      imparo_stream stream) {
+    if (!in || !w_t || !out || n_tokens < 0 || heads < 1 || k < 8 || n < 1) return IMPARO_BAD_ARGUMENT;
+    if (k % 8 || in_ld % 8 || in_hs % 8) return IMPARO_BAD_ARGUMENT;
+    if (in_hs < k || in_ld < (heads - 1) * in_hs + k || out_hs < n || out_ld < (heads - 1) * out_hs + n)
+        return IMPARO_BAD_ARGUMENT;
+    if (n_tokens == 0) return IMPARO_OK;
+    const int n_tiles = (n + 15) / 16;
+    const dim3 grid((n_tokens + 15) / 16, heads, (n_tiles + LAT_WAVES - 1) / LAT_WAVES);
+    if (grid.y > 65535 || grid.z > 65535) return IMPARO_BAD_ARGUMENT;
+    hipStream_t s = (hipStream_t)stream;
+    if (out_dtype == IMPARO_BF16)
+        k_head_gemm_tiles<bf16_t><<<grid, LAT_WAVES * WAVE, 0, s>>>((const bf16_t*)in, in_ld, in_hs, (const bf16_t*)w_t,
+                                                                   (bf16_t*)out, out_ld, out_hs, n_tokens, k, n);
+    else if (out_dtype == IMPARO_F32)
+        k_head_gemm_tiles<float><<<grid, LAT_WAVES * WAVE, 0, s>>>((const bf16_t*)in, in_ld, in_hs, (const bf16_t*)w_t,
+                                                                  (float*)out, out_ld, out_hs, n_tokens, k, n);
+    else
+        return IMPARO_BAD_ARGUMENT;
+    return launch_status();
+}
+
 // Asks the runtime about one kernel of this file, which makes it load the file's code onto the
 // current device (a stream under capture cannot).
 int imparo_load_code_latent_attention() {

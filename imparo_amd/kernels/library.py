@@ -78,7 +78,8 @@ _SIGNATURES = {
     "imparo_attention_latent_tiles_split": [I, I, I, P],
     "imparo_attention_latent_tiles": [P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, I, I, P],
     "imparo_head_gemm": [P, I, I, P, I, P, I, I, I, I, I, I, I, P],
-    "imparo_hgrn2_scan": [P, I, I, I, I, P, P, P, P, P, P, I, I, I, I, P],
+    "imparo_head_gemm_tiles": [P, I, I, P, P, I, I, I, I, I, I, I, P],
+    "imparo_hgrn2_scan": [P, I, I, I, I, P, P, P, P, P, P, I, I, I, I, I, I, P, P, P],
     "imparo_gated_sum": [P, P, I, P, I, P, I, P, I, I, I, P],
     "imparo_side_gate": [P, P, I, I, I, P, I, P, I, I, I, I, P],
     "imparo_add_rows": [P, P, c_int64, P],

@@ -952,6 +952,27 @@ def head_gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, out_columns: 
     return out
 
 
+def head_gemm_tiles_takes(dtype: torch.dtype, k: int) -> bool:
+    """Whether the matrix-core form of the per-head product takes inputs of this dtype and inner size."""
+    return dtype == torch.bfloat16 and k >= 8 and k % 8 == 0
+
+
+def head_gemm_tiles(x: torch.Tensor, w_t: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """head_gemm on the matrix cores: x [tokens, heads, k] bfloat16, w_t [heads, n, k] bfloat16 (a head's matrix
+    with the inner size running fastest); out [tokens, heads, at least n] bfloat16 or float32."""
+    T, H, K = x.shape
+    Hw, N, Kw = w_t.shape
+    if (Hw, Kw) != (H, K) or not head_gemm_tiles_takes(x.dtype, K) or w_t.dtype != torch.bfloat16:
+        raise KernelArgumentError(f"head_gemm_tiles: x is {tuple(x.shape)} {x.dtype}, the weights {tuple(w_t.shape)} {w_t.dtype}")
+    if out.dim() != 3 or out.shape[0] != T or out.shape[1] != H or out.shape[2] < N:
+        raise KernelArgumentError(f"head_gemm_tiles: out is {tuple(out.shape)}; [{T}, {H}, at least {N}] is needed")
+    _check(library().imparo_head_gemm_tiles(
+        _dev(x, "head_gemm x", torch.bfloat16), H * K, K, _dev(w_t, "head_gemm weights", torch.bfloat16),
+        _dev(out, "head_gemm out"), _code(out, "head_gemm out"), H * out.shape[2], out.shape[2], T, H, K, N, _stream()),
+        "head_gemm_tiles")
+    return out
+
+
 def attention_latent(q: torch.Tensor, cache: torch.Tensor, out: torch.Tensor, positions: torch.Tensor,
                      row_of_token: torch.Tensor, block_table: torch.Tensor, value_dim: int, scale: float,
                      window: Optional[int]) -> torch.Tensor:
@@ -1020,19 +1041,40 @@ def attention_latent_tiles(q: torch.Tensor, cache: torch.Tensor, cache_t: torch.
 # ---------------------------------------------------------------- gated linear recurrence
 def hgrn2_scan(rows: torch.Tensor, q_off: int, f_off: int, v_off: int, lower: torch.Tensor, state: torch.Tensor,
                seg_start: torch.Tensor, seg_len: torch.Tensor, slot: torch.Tensor, out: torch.Tensor, heads: int,
-               dim: int, vdim: int) -> torch.Tensor:
+               dim: int, vdim: int, chunk_tokens: int = 0, max_chunks: int = 0,
+               chunk_state: Optional[torch.Tensor] = None, chunk_decay: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Per request and head, token by token: S <- diag(f) S + (1 - f) v^T, out = S^T q with q = silu(zq),
-    f = lower + (1 - lower) sigmoid(zf); rows holds zq, zf, v at the given columns."""
+    f = lower + (1 - lower) sigmoid(zf); rows holds zq, zf, v at the given columns. With `chunk_tokens`
+    (hgrn2_chunks) segments are walked in chunks side by side: `max_chunks` bounds the chunks of the longest,
+    `chunk_state` (rows * max_chunks * heads * dim * vdim) and `chunk_decay` (rows * max_chunks * heads * dim)
+    float32 are scratch."""
     n, ld = rows.shape
     R = seg_start.shape[0]
+    if chunk_tokens:
+        if (chunk_state is None or chunk_decay is None or chunk_state.numel() < R * max_chunks * heads * dim * vdim
+                or chunk_decay.numel() < R * max_chunks * heads * dim):
+            raise KernelArgumentError("hgrn2_scan: the scratch for the chunks is missing or too small")
+        _dev(chunk_state, "chunk states", torch.float32)
+        _dev(chunk_decay, "chunk decays", torch.float32)
     _check(library().imparo_hgrn2_scan(
         _dev(rows, "recurrence inputs", torch.float32), ld, q_off, f_off, v_off,
         _dev(lower, "lower bounds", torch.float32, (heads * dim,)),
         _dev(state, "recurrent state", torch.float32, (state.shape[0], heads, dim, vdim)),
         _dev(seg_start, "seg_start", torch.int32, (R,)), _dev(seg_len, "seg_len", torch.int32, (R,)),
         _dev(slot, "slot", torch.int32, (R,)), _dev(out, "recurrence out", torch.float32, (n, heads * vdim)),
-        R, heads, dim, vdim, _stream()), "hgrn2_scan")
+        R, heads, dim, vdim, int(chunk_tokens), int(max_chunks),
+        chunk_state.data_ptr() if chunk_tokens else None, chunk_decay.data_ptr() if chunk_tokens else None,
+        _stream()), "hgrn2_scan")
     return out
+
+
+def hgrn2_chunks(max_seg_len: int):
+    """(tokens a chunk, chunks of the longest segment) for a step whose longest segment has `max_seg_len`
+    tokens; (0, 0): too short to pay for three launches. At most 32 chunks a segment."""
+    if max_seg_len < 256:
+        return 0, 0
+    tokens = max(128, (-(-max_seg_len // 32) + 7) // 8 * 8)
+    return tokens, -(-max_seg_len // tokens)
 
 
 # ---------------------------------------------------------------- a parallel block's elementwise pieces

@@ -84,8 +84,14 @@ class Hgrn2:
         T, H, dk, dv = h.shape[0], self.heads, self.dim, self.vdim
         rows = self.proj(ctx, h, torch.float32, "hgrn2_rows", alias="mixer_in")
         o = ctx.workspace.get("hgrn2_out", (T, H * dv), torch.float32)
+        chunk_tokens, max_chunks = ops.hgrn2_chunks(ctx.max_seg_len)
+        chunk_state = chunk_decay = None
+        if chunk_tokens:
+            # a long portion: its chunks side by side, each from the state that a pass over the chunks' ends leaves it
+            chunk_state = ctx.workspace.get("hgrn2_chunk_state", (ctx.seg_start.shape[0] * max_chunks * H * dk * dv,), torch.float32)
+            chunk_decay = ctx.workspace.get("hgrn2_chunk_decay", (ctx.seg_start.shape[0] * max_chunks * H * dk,), torch.float32)
         ops.hgrn2_scan(rows, 0, H * dk, 2 * H * dk, self.lower, ctx.fixed_arrays(site)["state"], ctx.seg_start,
-                       ctx.seg_len, ctx.slot, o, H, dk, dv)
+                       ctx.seg_len, ctx.slot, o, H, dk, dv, chunk_tokens, max_chunks, chunk_state, chunk_decay)
         normed = ctx.workspace.get("hgrn2_normed", (T, H * dv), self.out.in_dtype, alias="mixer_mid")
         ops.group_rms_norm(o, self.norm, H, self.eps, normed)
         return self.out(ctx, normed, torch.float32, "mixer_out", sliced_ok=True)

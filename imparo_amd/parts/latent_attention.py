@@ -95,8 +95,12 @@ class LatentAttention:
         self.kv_norm = place_vector(tensors[n["dkv_norm"]], device)
         # the two up-projections head by head, laid [heads, in, out] as the small product reads them:
         # W_uk[h] is [dim, rank] and maps dim -> rank as its transpose; W_uv[h] is [vdim, rank] and maps rank -> vdim
-        self.w_absorb = tensors[n["uk"]].reshape(H, dn, r).to(device=device, dtype=engine_dtype).contiguous()
-        self.w_values = tensors[n["uv"]].reshape(H, dv, r).transpose(1, 2).to(device=device, dtype=engine_dtype).contiguous()
+        # (the matrix-core form of that product wants them [heads, out, in], where it takes the sizes)
+        uk, uv = tensors[n["uk"]].reshape(H, dn, r), tensors[n["uv"]].reshape(H, dv, r)
+        self.absorb_tiles = ops.head_gemm_tiles_takes(engine_dtype, dn)
+        self.values_tiles = ops.head_gemm_tiles_takes(engine_dtype, r)
+        self.w_absorb = (uk.transpose(1, 2) if self.absorb_tiles else uk).to(device=device, dtype=engine_dtype).contiguous()
+        self.w_values = (uv if self.values_tiles else uv.transpose(1, 2)).to(device=device, dtype=engine_dtype).contiguous()
         self.out = Linear(place_projection(tensors[n["o"]], engine_dtype, device))
         pos = spec.get("position") or PartSpec("none")
         self.position = part_class("position", pos.kind)(pos, device)
@@ -137,7 +141,8 @@ class LatentAttention:
                          table if owns_cache else None, ctx.page_size, cache if owns_cache else None,
                          q_plain, q_full, H, self.dim, self.rot_dim, self.rank,
                          cache_t=arrays["latent_t"] if self.tiles and owns_cache else None)
-        ops.head_gemm(q_plain, self.w_absorb, q_full)               # columns 0 .. rank of every head's query
+        # columns 0 .. rank of every head's query
+        (ops.head_gemm_tiles if self.absorb_tiles else ops.head_gemm)(q_plain, self.w_absorb, q_full)
         mixed = ws.get("latent_mixed", (T, H * self.rank), ctx.dtype, alias="mixer_mid")
         if self.tiles:
             n_splits, split_keys = ops.attention_latent_tiles_split(T, H, ctx.max_context)
@@ -151,7 +156,7 @@ class LatentAttention:
             ops.attention_latent(q_full, cache, mixed, ctx.positions, ctx.row_of_token, table, self.rank, self.scale,
                                  self.window)
         o = ws.get("latent_values", (T, H, self.vdim), self.out.in_dtype)
-        ops.head_gemm(mixed.view(T, H, self.rank), self.w_values, o)
+        (ops.head_gemm_tiles if self.values_tiles else ops.head_gemm)(mixed.view(T, H, self.rank), self.w_values, o)
         return self.out(ctx, o.view(T, H * self.vdim), torch.float32, "mixer_out", sliced_ok=True)
 
 

@@ -112,10 +112,12 @@ def plain_recurrence(zq, zf, v, low, S):
     return out, S
 
 
+@pytest.mark.parametrize("chunk", [0, 8, 16])
 @pytest.mark.parametrize("H,dk,dv", [(2, 16, 24), (3, 20, 12), (1, 1, 1), (2, 128, 64), (1, 200, 300), (4, 32, 64)])
-def test_recurrence_kernel_continues_over_segments_in_used_slots(H, dk, dv):
+def test_recurrence_kernel_continues_over_segments_in_used_slots(H, dk, dv, chunk):
     """Three requests in slots 5, 0, 2 (two of them left dirty by an earlier request), fed in segments of
-    1, 2, 19 and 77 tokens in changing company: each equals the recurrence over its whole sequence."""
+    1, 2, 19 and 77 tokens in changing company: each equals the recurrence over its whole sequence. Also with
+    the segments walked in chunks of `chunk` tokens side by side (segments of one chunk and of ten)."""
     from imparo_amd.kernels import ops
     g = torch.Generator().manual_seed(dk)
     lengths, slots = [99, 40, 3], [5, 0, 2]
@@ -139,8 +141,10 @@ def test_recurrence_kernel_continues_over_segments_in_used_slots(H, dk, dv):
                 fed[r] += k
         start = np.cumsum([0] + [k for _, k in segs])[:-1]
         out = torch.empty(sum(k for _, k in segs), H * dv, device=DEV)
+        chunks = -(-max(k for _, k in segs) // chunk) if chunk else 0
+        scratch = [torch.full((len(segs) * chunks * H * dk * d,), float("nan"), device=DEV) for d in (dv, 1)] if chunk else [None, None]
         ops.hgrn2_scan(dev(torch.cat(rows)), 0, H * dk, 2 * H * dk, dev(low.reshape(-1)), state, i32(start),
-                       i32([k for _, k in segs]), i32([slots[r] for r, _ in segs]), out, H, dk, dv)
+                       i32([k for _, k in segs]), i32([slots[r] for r, _ in segs]), out, H, dk, dv, chunk, chunks, *scratch)
         assert width == rows[0].shape[1]
         for (r, k), s0 in zip(segs, start):
             got[r].append(out[s0:s0 + k].cpu())
@@ -220,6 +224,21 @@ def test_latent_attention_kernel(H, r, dr, page, window, dtype):
     """A portion behind cached rows beside single tokens and a fresh prompt, in shuffled pages."""
     got, want = latent_case(H, r, dr, [(37, 21), (90, 1), (0, 70), (15, 1)], page, dtype, window)
     close(got, want, dtype, "attention over shared rows")
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("T,H,K,N,wide", [(1, 2, 8, 5, 0), (37, 3, 24, 40, 8), (16, 1, 64, 256, 32), (130, 5, 136, 17, 3), (8, 33, 256, 64, 0)])
+def test_head_product_on_the_matrix_cores(T, H, K, N, wide, out_dtype):
+    """Inner sizes that fill a product of 32 and that do not, outputs that end inside a tile, rows wider than a head's outputs."""
+    from imparo_amd.kernels import ops
+    g = torch.Generator().manual_seed(T + K)
+    x = torch.randn(T, H, K, generator=g).to(torch.bfloat16)
+    w = torch.randn(H, N, K, generator=g).to(torch.bfloat16)
+    out = torch.full((T, H, N + wide), 7.0, dtype=out_dtype, device=DEV)
+    ops.head_gemm_tiles(dev(x, torch.bfloat16), dev(w, torch.bfloat16), out)
+    want = torch.einsum("thk,hnk->thn", x.float(), w.float())
+    close(out[:, :, :N], want, out_dtype if out_dtype == torch.bfloat16 else torch.float32, "per-head product, tiled")
+    assert float((out[:, :, N:].float() - 7.0).abs().max()) == 0.0 if wide else True
 
 
 @pytest.mark.parametrize("split_keys", [None, 32, 64])
@@ -393,6 +412,29 @@ def test_portions_of_changing_size(dirs, plains, name, page, dtype):
         eng = make_engine(dirs[name], dtype, page_size=page, use_graphs=graphs)
         got = step_all(eng, "p", tokens if cuts != (1,) else tokens[:45], cuts)
         check(got, ref[:got.shape[0]], dtype, f"{name} cuts {cuts}", bound(dtype, runs(name)))
+
+
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_a_long_portion_beside_a_short_one(dirs, plains, name):
+    """Portions of 300 and 290 tokens (the recurrence walks such a step in chunks side by side) beside one of 3
+    and a single token, then the rest: every request's logits are those of its whole prompt."""
+    from imparo_amd.engine import StepEntry
+    prompts = [prompt_tokens(vocab(name), n, 40 + i) for i, n in enumerate((330, 300, 9, 5))]
+    eng = make_engine(dirs[name], "float32", page_size=16)
+    cuts = [(300, 30), (290, 10), (3, 6), (1, 4)]
+    got = [[] for _ in prompts]
+    for step in range(2):
+        entries = []
+        for i, p in enumerate(prompts):
+            lo = sum(cuts[i][:step])
+            entries.append(StepEntry(i, p[lo:lo + cuts[i][step]], list(range(cuts[i][step]))))
+        out = eng.step(entries).cpu()
+        at = 0
+        for i, e in enumerate(entries):
+            got[i].append(out[at:at + len(e.tokens)])
+            at += len(e.tokens)
+    for i, p in enumerate(prompts):
+        check(torch.cat(got[i]), plains[name].logits(p), "float32", f"{name} request {i}", bound("float32", runs(name)))
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
