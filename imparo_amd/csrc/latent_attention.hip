@@ -8,6 +8,8 @@
 //   head_gemm     out[t, h, :] = W[h] in[t, h, :], a small product per head (the two absorbed
 //                 up-projections), float32 sums in the order k = 0, 1, 2, ...
 #include "common.h"
+
+#include <algorithm>
 #include "api.h"
 
 #define LAT_MAX_FREQ 256
@@ -161,7 +163,8 @@ extern "C" int imparo_head_gemm(const void* in, int in_ld, int in_hs, const void
 }
 
 // ---------------------------------------------------------------- the matrix-core kernel
-// A wave takes up to 16 heads of one token as the 16 queries of its products: every head reads the same
+// A wave takes up to 16 heads of one token as the 16 queries of its products (32 heads, as two such sets, where
+// a token has more than 16: every loaded tile then feeds twice the products): every head reads the same
 // rows, so one tile of keys serves them all, and they share one range of keys. Keys are walked in tiles of
 // 32 at absolute multiples of 32:
 //   S^T[key][head] = rows . Q^T     A = 16 bytes of a cached row a lane, B = Q^T in registers. Row m of
@@ -181,13 +184,11 @@ union LatFrag {
 
 #define LAT_WAVES 4
 
-__device__ __forceinline__ uint32_t lat_pack2(float a, float b) {
-    return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
-}
+__device__ __forceinline__ uint32_t lat_pack2(float a, float b) { return f32x2_to_bf16x2(a, b); }
 
 __device__ __forceinline__ float lat_bf16_value(float a) { return __uint_as_float((uint32_t)f32_to_bf16(a) << 16); }
 
-template <int NK, int NV>
+template <int NK, int NV, int QT>
 __global__ __launch_bounds__(LAT_WAVES * WAVE) void k_latent_attention_tiles(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ rows, const bf16_t* __restrict__ rows_t,
     bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
@@ -196,15 +197,14 @@ __global__ __launch_bounds__(LAT_WAVES * WAVE) void k_latent_attention_tiles(
     int row_dim, int rank, float scale, int window, int split_keys, int n_splits, int exact) {
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
     const int c = lane & 15, g = lane >> 4;
-    const int head_groups = (heads + 15) / 16;
+    const int head_groups = (heads + 16 * QT - 1) / (16 * QT);
     const long long total = (long long)n_tokens * head_groups * n_splits;
     const long long id = (long long)blockIdx.x * LAT_WAVES + wave;
     if (id >= total) return;                       // (no barrier below: waves are on their own)
     const int split = (int)(id % n_splits);
     const long long rest = id / n_splits;
     const int t = (int)(rest % n_tokens);
-    const int h = (int)(rest / n_tokens) * 16 + c;  // this lane's head
-    const bool live = h < heads;
+    const int h0 = (int)(rest / n_tokens) * 16 * QT + c;   // this lane's heads: h0, h0 + 16, ...
     const int pos = positions[t];
     const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
     const int k_lo = n_splits > 1 ? max(lo, split * split_keys) : lo;
@@ -212,19 +212,24 @@ __global__ __launch_bounds__(LAT_WAVES * WAVE) void k_latent_attention_tiles(
     const int page_size = 1 << page_shift, page_mask = page_size - 1;
     const int32_t* table = block_table + (size_t)row_of_token[t] * table_stride;
 
-    LatFrag qf[NK];
-    {
+    LatFrag qf[QT][NK];
+    lat_f32x4 o[QT][NV];
+    float m[QT], l[QT];
+#pragma unroll
+    for (int u = 0; u < QT; ++u) {
+        const int h = h0 + 16 * u;
+        const bool live = h < heads;
         const bf16_t* qrow = q + ((size_t)t * heads + (live ? h : 0)) * row_dim;
 #pragma unroll
         for (int dk = 0; dk < NK; ++dk) {
             const int d0 = dk * 32 + 8 * g;
-            qf[dk].u = (live && d0 < row_dim) ? *reinterpret_cast<const uint4*>(qrow + d0) : make_uint4(0u, 0u, 0u, 0u);
+            qf[u][dk].u = (live && d0 < row_dim) ? *reinterpret_cast<const uint4*>(qrow + d0) : make_uint4(0u, 0u, 0u, 0u);
         }
-    }
-    lat_f32x4 o[NV];
 #pragma unroll
-    for (int dt = 0; dt < NV; ++dt) o[dt] = lat_f32x4{0.f, 0.f, 0.f, 0.f};
-    float m = -INFINITY, l = 0.f;
+        for (int dt = 0; dt < NV; ++dt) o[u][dt] = lat_f32x4{0.f, 0.f, 0.f, 0.f};
+        m[u] = -INFINITY;
+        l[u] = 0.f;
+    }
 
     if (k_lo <= k_hi) {
         for (int base = k_lo & ~31; base <= k_hi; base += 32) {
@@ -248,36 +253,17 @@ __global__ __launch_bounds__(LAT_WAVES * WAVE) void k_latent_attention_tiles(
                 for (int dt = 0; dt < NV; ++dt)
                     vf[dt].u = *reinterpret_cast<const uint4*>(vbase + (size_t)min(dt * 16 + c, rank - 1) * page_size);
             }
-            lat_f32x4 s[2];
+            lat_f32x4 s[QT][2];
 #pragma unroll
             for (int t2 = 0; t2 < 2; ++t2) {
-                s[t2] = lat_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int u = 0; u < QT; ++u) s[u][t2] = lat_f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int dk = 0; dk < NK; ++dk)
-                    s[t2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t2][dk].v, qf[dk].v, s[t2], 0, 0, 0);
-            }
-            float sv[8];
-            float tile_max = -INFINITY;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int key = kg + j;
-                sv[j] = (key >= k_lo && key <= k_hi) ? s[j >> 2][j & 3] * scale : -INFINITY;
-                tile_max = fmaxf(tile_max, sv[j]);
+                    for (int u = 0; u < QT; ++u)
+                        s[u][t2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t2][dk].v, qf[u][dk].v, s[u][t2], 0, 0, 0);
             }
-            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE));
-            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE));
-            const float m_new = fmaxf(m, tile_max);  // finite: every tile holds a key of the range
-            const float corr = expf(m - m_new);
-            float p[8], p_sum = 0.f;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                p[j] = expf(sv[j] - m_new);
-                p_sum += p[j];
-            }
-            l = l * corr + p_sum;                   // a lane's own 8 keys; the four lanes of a head are added at the end
-            m = m_new;
-#pragma unroll
-            for (int dt = 0; dt < NV; ++dt) o[dt] *= corr;
             if (base < k_lo || base + 31 > k_hi) {  // what a page holds beyond the range may be anything: zeros instead
                 uint32_t keep[4];
 #pragma unroll
@@ -290,49 +276,81 @@ __global__ __launch_bounds__(LAT_WAVES * WAVE) void k_latent_attention_tiles(
                 for (int dt = 0; dt < NV; ++dt)
                     vf[dt].u = make_uint4(vf[dt].u.x & keep[0], vf[dt].u.y & keep[1], vf[dt].u.z & keep[2], vf[dt].u.w & keep[3]);
             }
-            LatFrag ph;
-            ph.u = make_uint4(lat_pack2(p[0], p[1]), lat_pack2(p[2], p[3]), lat_pack2(p[4], p[5]), lat_pack2(p[6], p[7]));
 #pragma unroll
-            for (int dt = 0; dt < NV; ++dt)
-                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, ph.v, o[dt], 0, 0, 0);
-            if (exact) {
-                float r[8];
+            for (int u = 0; u < QT; ++u) {
+                float sv[8];
+                float tile_max = -INFINITY;
 #pragma unroll
-                for (int j = 0; j < 8; ++j) r[j] = p[j] - lat_bf16_value(p[j]);
-                LatFrag pl;
-                pl.u = make_uint4(lat_pack2(r[0], r[1]), lat_pack2(r[2], r[3]), lat_pack2(r[4], r[5]), lat_pack2(r[6], r[7]));
+                for (int j = 0; j < 8; ++j) {
+                    const int key = kg + j;
+                    sv[j] = (key >= k_lo && key <= k_hi) ? s[u][j >> 2][j & 3] * scale : -INFINITY;
+                    tile_max = fmaxf(tile_max, sv[j]);
+                }
+                tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, WAVE));
+                tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE));
+                const float m_new = fmaxf(m[u], tile_max);  // finite: every tile holds a key of the range
+                const float corr = __expf(m[u] - m_new);
+                float p[8], p_sum = 0.f;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    p[j] = __expf(sv[j] - m_new);
+                    p_sum += p[j];
+                }
+                l[u] = l[u] * corr + p_sum;         // a lane's own 8 keys; the four lanes of a head are added at the end
+                if (__builtin_amdgcn_ballot_w64(m_new != m[u])) {   // (no head's maximum moved: every factor is 1)
+#pragma unroll
+                    for (int dt = 0; dt < NV; ++dt) o[u][dt] *= corr;
+                }
+                m[u] = m_new;
+                LatFrag ph;
+                ph.u = make_uint4(lat_pack2(p[0], p[1]), lat_pack2(p[2], p[3]), lat_pack2(p[4], p[5]), lat_pack2(p[6], p[7]));
 #pragma unroll
                 for (int dt = 0; dt < NV; ++dt)
-                    o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pl.v, o[dt], 0, 0, 0);
+                    o[u][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, ph.v, o[u][dt], 0, 0, 0);
+                if (exact) {
+                    float r[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) r[j] = p[j] - lat_bf16_value(p[j]);
+                    LatFrag pl;
+                    pl.u = make_uint4(lat_pack2(r[0], r[1]), lat_pack2(r[2], r[3]), lat_pack2(r[4], r[5]), lat_pack2(r[6], r[7]));
+#pragma unroll
+                    for (int dt = 0; dt < NV; ++dt)
+                        o[u][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pl.v, o[u][dt], 0, 0, 0);
+                }
             }
         }
     }
-    l += __shfl_xor(l, 16, WAVE);
-    l += __shfl_xor(l, 32, WAVE);
-    if (!live) return;
-    const size_t row = (size_t)t * heads + h;
-    if (n_splits == 1) {
-        const float inv = l > 0.f ? 1.0f / l : 0.f;
-        bf16_t* dst = out + row * rank;
 #pragma unroll
-        for (int dt = 0; dt < NV; ++dt)
+    for (int u = 0; u < QT; ++u) {
+        float lu = l[u];
+        lu += __shfl_xor(lu, 16, WAVE);
+        lu += __shfl_xor(lu, 32, WAVE);
+        const int h = h0 + 16 * u;
+        if (h >= heads) continue;
+        const size_t row = (size_t)t * heads + h;
+        if (n_splits == 1) {
+            const float inv = lu > 0.f ? 1.0f / lu : 0.f;
+            bf16_t* dst = out + row * rank;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int d = dt * 16 + 4 * g + i;
-                if (d < rank) dst[d] = f32_to_bf16(o[dt][i] * inv);
+            for (int dt = 0; dt < NV; ++dt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int d = dt * 16 + 4 * g + i;
+                    if (d < rank) dst[d] = f32_to_bf16(o[u][dt][i] * inv);
+                }
+        } else {
+            float* dst = part_o + (row * n_splits + split) * rank;
+#pragma unroll
+            for (int dt = 0; dt < NV; ++dt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int d = dt * 16 + 4 * g + i;
+                    if (d < rank) dst[d] = o[u][dt][i];
+                }
+            if (g == 0) {
+                part_ml[(row * n_splits + split) * 2] = m[u];
+                part_ml[(row * n_splits + split) * 2 + 1] = lu;
             }
-    } else {
-        float* dst = part_o + (row * n_splits + split) * rank;
-#pragma unroll
-        for (int dt = 0; dt < NV; ++dt)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int d = dt * 16 + 4 * g + i;
-                if (d < rank) dst[d] = o[dt][i];
-            }
-        if (g == 0) {
-            part_ml[(row * n_splits + split) * 2] = m;
-            part_ml[(row * n_splits + split) * 2 + 1] = l;
         }
     }
 }
@@ -378,8 +396,14 @@ extern "C" int imparo_attention_latent_tiles_takes(int row_dim, int rank, int pa
 
 // Into how many parts the keys of a launch are cut, and how many keys a part holds: few tokens over long
 // contexts would leave most of the chip idle. Parts lie at absolute multiples of their size.
+// 32 heads a wave where the launch fills the chip that way; few tokens are better spread over more waves.
+static int latent_heads_a_wave(int n_tokens, int heads) {
+    return heads > 16 && (long long)n_tokens * ((heads + 31) / 32) >= 512 ? 32 : 16;
+}
+
 extern "C" int imparo_attention_latent_tiles_split(int n_tokens, int heads, int max_context, int* split_keys) {
-    const long long items = (long long)n_tokens * ((heads + 15) / 16);
+    const int per = latent_heads_a_wave(n_tokens, heads);
+    const long long items = (long long)n_tokens * ((heads + per - 1) / per);
     int want = items >= 512 ? 1 : (int)((512 + items - 1) / items);
     int keys = ((max_context + want - 1) / want + 63) / 64 * 64;
     if (keys < 64) keys = 64;
@@ -388,15 +412,15 @@ extern "C" int imparo_attention_latent_tiles_split(int n_tokens, int heads, int 
     return n;
 }
 
-template <int NK, int NV>
+template <int NK, int NV, int QT>
 static void launch_latent_tiles(const void* q, const void* rows, const void* rows_t, void* out, float* part_o,
                                 float* part_ml, const int32_t* positions, const int32_t* row_of_token,
                                 const int32_t* block_table, int table_stride, int page_shift, int n_pages, int n_tokens,
                                 int heads, int row_dim, int rank, float scale, int window, int split_keys, int n_splits,
                                 int exact, hipStream_t s) {
-    const long long waves = (long long)n_tokens * ((heads + 15) / 16) * n_splits;
+    const long long waves = (long long)n_tokens * ((heads + 16 * QT - 1) / (16 * QT)) * n_splits;
     const unsigned blocks = (unsigned)((waves + LAT_WAVES - 1) / LAT_WAVES);
-    k_latent_attention_tiles<NK, NV><<<blocks, LAT_WAVES * WAVE, 0, s>>>(
+    k_latent_attention_tiles<NK, NV, QT><<<blocks, LAT_WAVES * WAVE, 0, s>>>(
         (const bf16_t*)q, (const bf16_t*)rows, (const bf16_t*)rows_t, (bf16_t*)out, part_o, part_ml, positions,
         row_of_token, block_table, table_stride, page_shift, n_pages, n_tokens, heads, row_dim, rank, scale, window,
         split_keys, n_splits, exact);
@@ -424,10 +448,16 @@ extern "C" int imparo_attention_latent_tiles(const void* q, const void* rows, co
     while ((1 << page_shift) < page_size) ++page_shift;
     hipStream_t s = (hipStream_t)stream;
 #define LAT_CASE(K, V)                                                                                               \
-    if (nk == K && nv == V)                                                                                          \
-        launch_latent_tiles<K, V>(q, rows, rows_t, out, part_o, part_ml, positions, row_of_token, block_table,       \
-                                  table_stride, page_shift, n_pages, n_tokens, heads, row_dim, rank, scale, window,  \
-                                  split_keys, n_splits, exact, s);
+    if (nk == K && nv == V) {                                                                                        \
+        if (latent_heads_a_wave(n_tokens, heads) == 32)                                                                       \
+            launch_latent_tiles<K, V, 2>(q, rows, rows_t, out, part_o, part_ml, positions, row_of_token, block_table, \
+                                         table_stride, page_shift, n_pages, n_tokens, heads, row_dim, rank, scale,    \
+                                         window, split_keys, n_splits, exact, s);                                    \
+        else                                                                                                         \
+            launch_latent_tiles<K, V, 1>(q, rows, rows_t, out, part_o, part_ml, positions, row_of_token, block_table, \
+                                         table_stride, page_shift, n_pages, n_tokens, heads, row_dim, rank, scale,    \
+                                         window, split_keys, n_splits, exact, s);                                    \
+    }
     LAT_CASE(2, 2) LAT_CASE(3, 2) LAT_CASE(3, 4) LAT_CASE(4, 4) LAT_CASE(5, 8) LAT_CASE(6, 8) LAT_CASE(9, 16) LAT_CASE(10, 16)
 #undef LAT_CASE
     if (launch_status() != IMPARO_OK) return IMPARO_LAUNCH_FAILED;
@@ -449,26 +479,27 @@ __global__ __launch_bounds__(LAT_WAVES * WAVE) void k_head_gemm_tiles(const bf16
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
     const int c = lane & 15, g = lane >> 4;
     const int h = blockIdx.y;
-    const int n_base = (blockIdx.z * LAT_WAVES + wave) * 16;
-    if (n_base >= N) return;
     const int token = blockIdx.x * 16 + c;
     const bool live = token < n_tokens;
-    const bf16_t* arow = w_t + ((size_t)h * N + min(n_base + c, N - 1)) * K;
     const bf16_t* brow = in + (size_t)(live ? token : 0) * in_ld + (size_t)h * in_hs;
-    lat_f32x4 acc = lat_f32x4{0.f, 0.f, 0.f, 0.f};
-    for (int k0 = 0; k0 < K; k0 += 32) {
-        const int kk = k0 + 8 * g;
-        LatFrag a, b;
-        a.u = kk < K ? *reinterpret_cast<const uint4*>(arow + kk) : make_uint4(0u, 0u, 0u, 0u);
-        b.u = (kk < K && live) ? *reinterpret_cast<const uint4*>(brow + kk) : make_uint4(0u, 0u, 0u, 0u);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc, 0, 0, 0);
-    }
-    if (!live) return;
-    TOut* dst = out + (size_t)token * out_ld + (size_t)h * out_hs;
+    TOut* dst = out + (size_t)(live ? token : 0) * out_ld + (size_t)h * out_hs;
+    // the launch's waves share a head's tiles of 16 outputs among them (many tokens: few, long-lived waves)
+    for (int n_base = (blockIdx.z * LAT_WAVES + wave) * 16; n_base < N; n_base += gridDim.z * LAT_WAVES * 16) {
+        const bf16_t* arow = w_t + ((size_t)h * N + min(n_base + c, N - 1)) * K;
+        lat_f32x4 acc = lat_f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int k0 = 0; k0 < K; k0 += 32) {
+            const int kk = k0 + 8 * g;
+            LatFrag a, b;
+            a.u = kk < K ? *reinterpret_cast<const uint4*>(arow + kk) : make_uint4(0u, 0u, 0u, 0u);
+            b.u = (kk < K && live) ? *reinterpret_cast<const uint4*>(brow + kk) : make_uint4(0u, 0u, 0u, 0u);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc, 0, 0, 0);
+        }
+        if (!live) continue;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int n = n_base + 4 * g + i;
-        if (n < N) store_f32<TOut>(dst, n, acc[i]);
+        for (int i = 0; i < 4; ++i) {
+            const int n = n_base + 4 * g + i;
+            if (n < N) store_f32<TOut>(dst, n, acc[i]);
+        }
     }
 }
 
@@ -483,7 +514,10 @@ extern "C" int imparo_head_gemm_tiles(const void* in, int in_ld, int in_hs, cons
         return IMPARO_BAD_ARGUMENT;
     if (n_tokens == 0) return IMPARO_OK;
     const int n_tiles = (n + 15) / 16;
-    const dim3 grid((n_tokens + 15) / 16, heads, (n_tiles + LAT_WAVES - 1) / LAT_WAVES);
+    const int all_z = (n_tiles + LAT_WAVES - 1) / LAT_WAVES;
+    const long long xy = (long long)((n_tokens + 15) / 16) * heads;
+    const int z = (int)std::min<long long>(all_z, std::max<long long>(1, (2048 + xy - 1) / xy));
+    const dim3 grid((n_tokens + 15) / 16, heads, z);
     if (grid.y > 65535 || grid.z > 65535) return IMPARO_BAD_ARGUMENT;
     hipStream_t s = (hipStream_t)stream;
     if (out_dtype == IMPARO_BF16)
