@@ -189,13 +189,14 @@ __device__ __forceinline__ uint32_t lat_pack2(float a, float b) { return f32x2_t
 __device__ __forceinline__ float lat_bf16_value(float a) { return __uint_as_float((uint32_t)f32_to_bf16(a) << 16); }
 
 template <int NK, int NV, int QT>
-__global__ __launch_bounds__(LAT_WAVES * WAVE) void k_latent_attention_tiles(
+__global__ __launch_bounds__(LAT_WAVES * WAVE, QT == 1 ? 2 : 1) void k_latent_attention_tiles(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ rows, const bf16_t* __restrict__ rows_t,
     bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ row_of_token,
     const int32_t* __restrict__ block_table, int table_stride, int page_shift, int n_pages, int n_tokens, int heads,
     int row_dim, int rank, float scale, int window, int split_keys, int n_splits, int exact) {
-    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+    // (what a wave shares is said to be the same in all of its lanes, so that it is kept and computed once a wave)
+    const int lane = threadIdx.x & (WAVE - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     const int c = lane & 15, g = lane >> 4;
     const int head_groups = (heads + 16 * QT - 1) / (16 * QT);
     const long long total = (long long)n_tokens * head_groups * n_splits;
@@ -233,11 +234,14 @@ __global__ __launch_bounds__(LAT_WAVES * WAVE) void k_latent_attention_tiles(
 
     if (k_lo <= k_hi) {
         for (int base = k_lo & ~31; base <= k_hi; base += 32) {
+            // a tile lies in one page (pages hold a multiple of 32 positions), and a part of it is in the range:
+            // addresses are held inside that part, so that no lane reads outside the tile's own page
+            const int page = min(max(table[base >> page_shift], 0), n_pages - 1);
+            const int t_lo = max(k_lo, base), t_hi = min(k_hi, base + 31);
             LatFrag kf[2][NK];
 #pragma unroll
             for (int t2 = 0; t2 < 2; ++t2) {
-                const int key = min(max(base + 8 * (c >> 2) + 4 * t2 + (c & 3), k_lo), k_hi);
-                const int page = min(max(table[key >> page_shift], 0), n_pages - 1);
+                const int key = min(max(base + 8 * (c >> 2) + 4 * t2 + (c & 3), t_lo), t_hi);
                 const bf16_t* krow = rows + ((size_t)page * page_size + (key & page_mask)) * row_dim;
 #pragma unroll
                 for (int dk = 0; dk < NK; ++dk)     // beyond the row: its last 8 again, against zeros of the query
@@ -246,8 +250,7 @@ __global__ __launch_bounds__(LAT_WAVES * WAVE) void k_latent_attention_tiles(
             const int kg = base + 8 * g;            // this lane's 8 keys in both products' results
             LatFrag vf[NV];
             {
-                const int kgc = min(max(kg, k_lo & ~7), k_hi & ~7);
-                const int page = min(max(table[kgc >> page_shift], 0), n_pages - 1);
+                const int kgc = min(max(kg, t_lo & ~7), t_hi & ~7);
                 const bf16_t* vbase = rows_t + (size_t)page * rank * page_size + (kgc & page_mask);
 #pragma unroll
                 for (int dt = 0; dt < NV; ++dt)
