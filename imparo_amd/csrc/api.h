@@ -137,8 +137,9 @@ int imparo_latent_store(const float* q_rows, const float* kv_rows, const float* 
 // The matrix-core form of imparo_attention_latent, bfloat16: up to 16 heads of a token are the 16 queries of a
 // wave's products. rows_t [pages, rank, page] holds the latents transposed inside a page; the values are the
 // latents (value_dim = rank). `_takes`: whether it is built for these sizes. `_split`: into how many parts the
-// keys are cut for this many tokens (and how many keys a part holds): with n_splits > 1, part_o [tokens, heads,
-// n_splits, rank] and part_ml [tokens, heads, n_splits, 2] float32 hold the parts, merged by a second launch.
+// keys are cut for this many tokens (and how many keys a part holds; 1 or a multiple of 4: a block adds the parts
+// of its four waves): with n_splits > 4, part_o [tokens, heads, n_splits / 4, rank] and part_ml [tokens, heads,
+// n_splits / 4, 2] float32 hold the blocks' sums, merged by a second launch.
 // `exact`: a softmax weight enters the product with the values as two bfloat16 numbers.
 int imparo_attention_latent_tiles_takes(int row_dim, int rank, int page_size);
 int imparo_attention_latent_tiles_split(int n_tokens, int heads, int max_context, int* split_keys);

@@ -201,7 +201,7 @@ __global__ __launch_bounds__(LAT_WAVES * WAVE, QT == 1 ? 2 : 1) void k_latent_at
     const int head_groups = (heads + 16 * QT - 1) / (16 * QT);
     const long long total = (long long)n_tokens * head_groups * n_splits;
     const long long id = (long long)blockIdx.x * LAT_WAVES + wave;
-    if (id >= total) return;                       // (no barrier below: waves are on their own)
+    if (id >= total) return;                       // (with parts the waves come in whole blocks: all reach the barrier below)
     const int split = (int)(id % n_splits);
     const long long rest = id / n_splits;
     const int t = (int)(rest % n_tokens);
@@ -323,6 +323,62 @@ __global__ __launch_bounds__(LAT_WAVES * WAVE, QT == 1 ? 2 : 1) void k_latent_at
             }
         }
     }
+    if (n_splits > 1) {
+        // The block's four waves hold four neighbouring parts of one token's keys (n_splits is a multiple of 4, and
+        // such launches take 16 heads a wave): waves 1 .. 3 leave theirs in LDS, wave 0 adds the four in order.
+        extern __shared__ float lat_parts[];         // [3][NV * 4 + 2][64]
+        constexpr int PER = (NV * 4 + 2) * WAVE;
+        float lu = l[0];
+        lu += __shfl_xor(lu, 16, WAVE);
+        lu += __shfl_xor(lu, 32, WAVE);
+        if (wave > 0) {
+            float* mine = lat_parts + (size_t)(wave - 1) * PER;
+#pragma unroll
+            for (int dt = 0; dt < NV; ++dt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) mine[(dt * 4 + i) * WAVE + lane] = o[0][dt][i];
+            mine[NV * 4 * WAVE + lane] = m[0];
+            mine[(NV * 4 + 1) * WAVE + lane] = lu;
+        }
+        __syncthreads();
+        if (wave > 0 || h0 >= heads) return;
+        float top = m[0], wt[LAT_WAVES];
+#pragma unroll
+        for (int w = 1; w < LAT_WAVES; ++w) top = fmaxf(top, lat_parts[(size_t)(w - 1) * PER + NV * 4 * WAVE + lane]);
+        wt[0] = m[0] == -INFINITY ? 0.f : __expf(m[0] - top);
+        float sum = wt[0] * lu;
+#pragma unroll
+        for (int w = 1; w < LAT_WAVES; ++w) {
+            const float mw = lat_parts[(size_t)(w - 1) * PER + NV * 4 * WAVE + lane];
+            wt[w] = mw == -INFINITY ? 0.f : __expf(mw - top);
+            sum += wt[w] * lat_parts[(size_t)(w - 1) * PER + (NV * 4 + 1) * WAVE + lane];
+        }
+        const int parts = n_splits / LAT_WAVES, part = split / LAT_WAVES;
+        const size_t row = (size_t)t * heads + h0;
+        const float inv = parts == 1 ? (sum > 0.f ? 1.0f / sum : 0.f) : 1.0f;
+#pragma unroll
+        for (int dt = 0; dt < NV; ++dt) {
+            const int d = dt * 16 + 4 * g;
+            float v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                v[i] = wt[0] * o[0][dt][i];
+#pragma unroll
+                for (int w = 1; w < LAT_WAVES; ++w) v[i] += wt[w] * lat_parts[(size_t)(w - 1) * PER + (dt * 4 + i) * WAVE + lane];
+                v[i] *= inv;
+            }
+            if (d >= rank) continue;                 // (rank is a multiple of 8: a lane's four numbers are in or out together)
+            if (parts == 1)
+                *reinterpret_cast<uint2*>(out + row * rank + d) = make_uint2(lat_pack2(v[0], v[1]), lat_pack2(v[2], v[3]));
+            else
+                *reinterpret_cast<float4*>(part_o + (row * parts + part) * rank + d) = make_float4(v[0], v[1], v[2], v[3]);
+        }
+        if (parts > 1 && g == 0) {
+            part_ml[(row * parts + part) * 2] = top;
+            part_ml[(row * parts + part) * 2 + 1] = sum;
+        }
+        return;
+    }
 #pragma unroll
     for (int u = 0; u < QT; ++u) {
         float lu = l[u];
@@ -330,53 +386,45 @@ __global__ __launch_bounds__(LAT_WAVES * WAVE, QT == 1 ? 2 : 1) void k_latent_at
         lu += __shfl_xor(lu, 32, WAVE);
         const int h = h0 + 16 * u;
         if (h >= heads) continue;
-        const size_t row = (size_t)t * heads + h;
-        if (n_splits == 1) {
-            const float inv = lu > 0.f ? 1.0f / lu : 0.f;
-            bf16_t* dst = out + row * rank;
+        const float inv = lu > 0.f ? 1.0f / lu : 0.f;
+        bf16_t* dst = out + ((size_t)t * heads + h) * rank;     // (rank is a multiple of 8: a lane's four numbers are in or out together)
 #pragma unroll
-            for (int dt = 0; dt < NV; ++dt)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int d = dt * 16 + 4 * g + i;
-                    if (d < rank) dst[d] = f32_to_bf16(o[u][dt][i] * inv);
-                }
-        } else {
-            float* dst = part_o + (row * n_splits + split) * rank;
-#pragma unroll
-            for (int dt = 0; dt < NV; ++dt)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int d = dt * 16 + 4 * g + i;
-                    if (d < rank) dst[d] = o[u][dt][i];
-                }
-            if (g == 0) {
-                part_ml[(row * n_splits + split) * 2] = m[u];
-                part_ml[(row * n_splits + split) * 2 + 1] = lu;
-            }
+        for (int dt = 0; dt < NV; ++dt) {
+            const int d = dt * 16 + 4 * g;
+            if (d < rank)
+                *reinterpret_cast<uint2*>(dst + d) = make_uint2(lat_pack2(o[u][dt][0] * inv, o[u][dt][1] * inv),
+                                                                lat_pack2(o[u][dt][2] * inv, o[u][dt][3] * inv));
         }
     }
 }
 
 // out[row, d] = sum_s w_s part_o[row, s, d] / sum_s w_s l_s with w_s = exp(m_s - max m), the parts in order.
+// A thread takes four neighbouring numbers of a row (rank is a multiple of 8).
 __global__ void k_latent_merge(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                bf16_t* __restrict__ out, long long n_rows, int n_splits, int rank) {
+    const int quads = rank / 4;
     const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n_rows * rank) return;
-    const long long row = i / rank;
-    const int d = (int)(i - row * rank);
+    if (i >= n_rows * quads) return;
+    const long long row = i / quads;
+    const int d = (int)(i - row * quads) * 4;
     const float* ml = part_ml + row * n_splits * 2;
     float top = -INFINITY;
     for (int s = 0; s < n_splits; ++s) top = fmaxf(top, ml[2 * s]);
-    float num = 0.f, den = 0.f;
+    float4 num = make_float4(0.f, 0.f, 0.f, 0.f);
+    float den = 0.f;
     for (int s = 0; s < n_splits; ++s) {
         const float ms = ml[2 * s];
         if (ms == -INFINITY) continue;
-        const float w = expf(ms - top);
-        num += w * part_o[(row * n_splits + s) * rank + d];
+        const float w = __expf(ms - top);
+        const float4 part = *reinterpret_cast<const float4*>(part_o + (row * n_splits + s) * rank + d);
+        num.x += w * part.x;
+        num.y += w * part.y;
+        num.z += w * part.z;
+        num.w += w * part.w;
         den += w * ml[2 * s + 1];
     }
-    out[i] = f32_to_bf16(den > 0.f ? num / den : 0.f);
+    const float inv = den > 0.f ? 1.0f / den : 0.f;
+    *reinterpret_cast<uint2*>(out + row * rank + d) = make_uint2(lat_pack2(num.x * inv, num.y * inv), lat_pack2(num.z * inv, num.w * inv));
 }
 
 // The sizes the matrix-core kernel is built for: latents of up to 256 numbers in steps of 8 (value tiles of
@@ -410,7 +458,8 @@ extern "C" int imparo_attention_latent_tiles_split(int n_tokens, int heads, int 
     int want = items >= 512 ? 1 : (int)((512 + items - 1) / items);
     int keys = ((max_context + want - 1) / want + 63) / 64 * 64;
     if (keys < 64) keys = 64;
-    const int n = max_context <= keys ? 1 : (max_context + keys - 1) / keys;
+    int n = max_context <= keys ? 1 : (max_context + keys - 1) / keys;
+    if (n > 1) n = (n + LAT_WAVES - 1) / LAT_WAVES * LAT_WAVES;    // a block's waves take neighbouring parts and add them
     if (split_keys) *split_keys = keys;
     return n;
 }
@@ -423,7 +472,8 @@ static void launch_latent_tiles(const void* q, const void* rows, const void* row
                                 int exact, hipStream_t s) {
     const long long waves = (long long)n_tokens * ((heads + 16 * QT - 1) / (16 * QT)) * n_splits;
     const unsigned blocks = (unsigned)((waves + LAT_WAVES - 1) / LAT_WAVES);
-    k_latent_attention_tiles<NK, NV, QT><<<blocks, LAT_WAVES * WAVE, 0, s>>>(
+    const size_t lds = n_splits > 1 ? (size_t)(LAT_WAVES - 1) * (NV * 4 + 2) * WAVE * sizeof(float) : 0;
+    k_latent_attention_tiles<NK, NV, QT><<<blocks, LAT_WAVES * WAVE, lds, s>>>(
         (const bf16_t*)q, (const bf16_t*)rows, (const bf16_t*)rows_t, (bf16_t*)out, part_o, part_ml, positions,
         row_of_token, block_table, table_stride, page_shift, n_pages, n_tokens, heads, row_dim, rank, scale, window,
         split_keys, n_splits, exact);
@@ -446,6 +496,7 @@ extern "C" int imparo_attention_latent_tiles(const void* q, const void* rows, co
         return IMPARO_BAD_ARGUMENT;
     if (n_splits < 1 || (n_splits > 1 && (!part_o || !part_ml || split_keys < 32 || split_keys % 32))) return IMPARO_BAD_ARGUMENT;
     if (n_splits > 1 && (long long)n_splits * split_keys > 0x7fffffffLL) return IMPARO_BAD_ARGUMENT;
+    if (n_splits > 1 && (n_splits % LAT_WAVES || latent_heads_a_wave(n_tokens, heads) != 16)) return IMPARO_BAD_ARGUMENT;
     if (n_tokens == 0) return IMPARO_OK;
     int page_shift = 0;
     while ((1 << page_shift) < page_size) ++page_shift;
@@ -464,10 +515,10 @@ extern "C" int imparo_attention_latent_tiles(const void* q, const void* rows, co
     LAT_CASE(2, 2) LAT_CASE(3, 2) LAT_CASE(3, 4) LAT_CASE(4, 4) LAT_CASE(5, 8) LAT_CASE(6, 8) LAT_CASE(9, 16) LAT_CASE(10, 16)
 #undef LAT_CASE
     if (launch_status() != IMPARO_OK) return IMPARO_LAUNCH_FAILED;
-    if (n_splits > 1) {
-        const long long n = (long long)n_tokens * heads * rank;
+    if (n_splits > LAT_WAVES) {
+        const long long n = (long long)n_tokens * heads * (rank / 4);
         k_latent_merge<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(part_o, part_ml, (bf16_t*)out, (long long)n_tokens * heads,
-                                                                  n_splits, rank);
+                                                                  n_splits / LAT_WAVES, rank);
     }
     return launch_status();
 }

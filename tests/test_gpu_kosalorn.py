@@ -199,6 +199,7 @@ def latent_case(H, r, dr, segments, page, dtype, window, boost=None, seed=0, til
         n_splits, keys = ops.attention_latent_tiles_split(T, H, longest)
         if split_keys is not None:
             n_splits, keys = -(-longest // split_keys), split_keys
+            n_splits = -(-n_splits // 4) * 4 if n_splits > 1 else 1          # (a block adds the parts of its four waves)
         part_o = torch.full((T * H * n_splits * r,), float("nan"), device=DEV)
         part_ml = torch.full((T * H * n_splits * 2,), float("nan"), device=DEV)
         cache_t = dev(cache[:, :, :r].transpose(1, 2), dtype)
