@@ -161,7 +161,7 @@ int imparo_head_gemm_tiles(const void* in, int in_ld, int in_hs, const void* w_t
 // ---- a gated linear recurrence with a matrix of state a head
 // Per request (row), head and token in order: q = silu(zq), f = lower + (1 - lower) sigmoid(zf),
 // S <- diag(f) S + (1 - f) v^T, out = S^T q. rows [tokens, ld] float32 holds zq at q_off, zf at f_off, v at v_off,
-// head by head; state [slots, heads, dim, vdim] float32; out [tokens, heads * vdim] float32. dim <= 256.
+// head by head; state [slots, heads, dim, vdim] float32; out [tokens, heads * vdim] float32. dim <= 512.
 // chunk_tokens 0: one launch, a block walks a row's whole segment. Otherwise (a multiple of 8) segments are walked
 // in chunks of that many tokens side by side, in three launches; max_chunks >= ceil(longest segment /
 // chunk_tokens); chunk_state [n_rows * max_chunks, heads, dim, vdim] and chunk_decay [n_rows * max_chunks, heads,

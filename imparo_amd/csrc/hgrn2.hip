@@ -22,7 +22,7 @@
 #define HG2_KPT 16            // entries of a column a thread keeps at most
 #define HG2_TOKENS 8          // tokens staged in LDS at once
 #define HG2_THREADS 256
-#define HG2_MAX_DIM 256
+#define HG2_MAX_DIM 512
 
 __device__ __forceinline__ float hg2_sigmoid(float z) { return 1.0f / (1.0f + expf(-z)); }
 
@@ -186,6 +186,7 @@ extern "C" int imparo_hgrn2_scan(const float* rows, int ld, int q_off, int f_off
         case 4: HG2_LAUNCH(4); break;
         case 8: HG2_LAUNCH(8); break;
         case 16: HG2_LAUNCH(16); break;
+        case 32: HG2_LAUNCH(32); break;
         default: return IMPARO_BAD_ARGUMENT;
     }
 #undef HG2_LAUNCH

@@ -17,7 +17,7 @@ from .library import library
 
 F32, BF16 = 0, 1
 ATTENTION_MAX_HEAD_DIM = 576      # the wave attention kernel's longest key row
-HGRN2_MAX_DIM = 256               # state rows a head of the gated linear recurrence
+HGRN2_MAX_DIM = 512               # state rows a head of the gated linear recurrence
 _CODES = {torch.float32: F32, torch.bfloat16: BF16}
 
 

@@ -113,7 +113,7 @@ def plain_recurrence(zq, zf, v, low, S):
 
 
 @pytest.mark.parametrize("chunk", [0, 8, 16])
-@pytest.mark.parametrize("H,dk,dv", [(2, 16, 24), (3, 20, 12), (1, 1, 1), (2, 128, 64), (1, 200, 300), (4, 32, 64)])
+@pytest.mark.parametrize("H,dk,dv", [(2, 16, 24), (3, 20, 12), (1, 1, 1), (2, 128, 64), (1, 200, 300), (4, 32, 64), (1, 330, 20), (2, 512, 8)])
 def test_recurrence_kernel_continues_over_segments_in_used_slots(H, dk, dv, chunk):
     """Three requests in slots 5, 0, 2 (two of them left dirty by an earlier request), fed in segments of
     1, 2, 19 and 77 tokens in changing company: each equals the recurrence over its whole sequence. Also with
