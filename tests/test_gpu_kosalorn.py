@@ -253,6 +253,14 @@ def test_latent_attention_on_the_matrix_cores(H, r, dr, page, window, split_keys
     close(got, want, torch.bfloat16, "attention over shared rows, tiled")
 
 
+@pytest.mark.parametrize("H,r,dr,page,window", [(33, 64, 32, 64, None), (40, 72, 8, 64, 100), (64, 256, 32, 64, 33), (17, 200, 24, 32, None)])
+def test_latent_attention_on_the_matrix_cores_many_tokens(H, r, dr, page, window):
+    """A launch large enough that a wave takes 32 heads (two sets of 16, the last one partly empty): two long
+    portions, one of them behind cached rows; latents that end inside a value tile and rows inside a product of 32."""
+    got, want = latent_case(H, r, dr, [(0, 300), (37, 230)], page, torch.bfloat16, window, tiles=True)
+    close(got, want, torch.bfloat16, "attention over shared rows, tiled, 32 heads a wave")
+
+
 @pytest.mark.parametrize("n_last", [1, 5])
 @pytest.mark.parametrize("window,page", [(24, 32), (64, 64), (65, 64), (33, 32), (1, 32), (32, 128)])
 def test_a_key_at_the_windows_edge_on_the_matrix_cores(window, page, n_last):
