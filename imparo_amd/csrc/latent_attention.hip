@@ -537,6 +537,7 @@ __global__ __launch_bounds__(LAT_WAVES * WAVE) void k_head_gemm_tiles(const bf16
     const bool live = token < n_tokens;
     const bf16_t* brow = in + (size_t)(live ? token : 0) * in_ld + (size_t)h * in_hs;
     TOut* dst = out + (size_t)(live ? token : 0) * out_ld + (size_t)h * out_hs;
+    const bool quads = out_ld % 4 == 0 && out_hs % 4 == 0;      // every head's outputs start where four of them align
     // the launch's waves share a head's tiles of 16 outputs among them (many tokens: few, long-lived waves)
     for (int n_base = (blockIdx.z * LAT_WAVES + wave) * 16; n_base < N; n_base += gridDim.z * LAT_WAVES * 16) {
         const bf16_t* arow = w_t + ((size_t)h * N + min(n_base + c, N - 1)) * K;
@@ -549,11 +550,17 @@ __global__ __launch_bounds__(LAT_WAVES * WAVE) void k_head_gemm_tiles(const bf16
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc, 0, 0, 0);
         }
         if (!live) continue;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int n = n_base + 4 * g + i;
-            if (n < N) store_f32<TOut>(dst, n, acc[i]);
+        const int n0 = n_base + 4 * g;
+        if (quads && n0 + 3 < N) {                   // a lane's four outputs in one store
+            if constexpr (sizeof(TOut) == 2)
+                *reinterpret_cast<uint2*>(dst + n0) = make_uint2(lat_pack2(acc[0], acc[1]), lat_pack2(acc[2], acc[3]));
+            else
+                *reinterpret_cast<float4*>(dst + n0) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+            continue;
         }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (n0 + i < N) store_f32<TOut>(dst, n0 + i, acc[i]);
     }
 }
 
