@@ -323,7 +323,7 @@ def test_latent_store_and_head_product(H, dn, dr, r, dims, pairs, n, dtype):
     page, p0 = 16, 70000 - n // 2
     q_rows, kv_rows = torch.randn(n, H * (dn + dr), generator=g), torch.randn(n, r + dr, generator=g)
     w = 0.5 + torch.rand(r, generator=g)
-    freq = plain.frequencies(dims, 250000.0, torch.float32) if dims else None
+    freq = plain.frequencies(dims, 300000.0, torch.float32) if dims else None
     pos = torch.arange(p0, p0 + n)
     n_pages = (p0 + n) // page + 1
     table = np.arange(n_pages, dtype=np.int32)[None, :]
