@@ -204,7 +204,7 @@ __global__ __launch_bounds__(LAT_WAVES * WAVE, QT == 1 ? 2 : 1) void k_latent_at
     if (id >= total) return;                       // (with parts the waves come in whole blocks: all reach the barrier below)
     const int split = (int)(id % n_splits);
     const long long rest = id / n_splits;
-    const int t = (int)(rest % n_tokens);
+    const int t = n_tokens - 1 - (int)(rest % n_tokens);    // late tokens of a prompt, with the most keys, start first
     const int h0 = (int)(rest / n_tokens) * 16 * QT + c;   // this lane's heads: h0, h0 + 16, ...
     const int pos = positions[t];
     const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
