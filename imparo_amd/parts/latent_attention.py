@@ -16,6 +16,15 @@ rotated part and a score is one dot product with a cached row; the softmax
 weights sum the cached latents, and W_uv is applied to that sum, once a query
 instead of once a key.
 
+Kernels: under a bfloat16 engine, with pages of at least 32 positions and a
+latent of up to 256 numbers in steps of 8, attention runs on the matrix cores,
+16 or 32 heads of one token a wave (all heads read the same rows over the same
+range of keys); the cache then keeps the latents a second time, transposed
+inside a page (`latent_t` [kv_rank, PAGE]), which is what the second product
+reads 8 positions at a time. Otherwise one wave a (token, head) walks the rows.
+Both per-head products run on the matrix cores where their inner sizes are
+multiples of 8.
+
 Parameters: width, heads, dim, rot_dim, vdim, kv_rank, q_rank (None: queries
 projected directly), scale, window (a query at position i sees positions
 i - window + 1 .. i; None: all before it), eps (of the latents' norms),
