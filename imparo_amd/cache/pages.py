@@ -112,15 +112,20 @@ class PagedSpec:
     """State that grows with the context, in pages: the arrays a mixer keeps
     per position (keys and values, a latent, whatever it declares), laid out
     as the mixer's kernels read them. `window` None keeps every position; a
-    number keeps only that many. Sites with equal specs share a pool and a
+    number keeps only that many. `chunk`: a query reads the positions of its
+    own chunk only (chunks of that many positions, counted from position 0),
+    so the pages of earlier chunks are given back. Sites with equal specs share a pool and a
     block table per request. `fixed`: what the site keeps per request beside
     its pages, of a fixed size (the input its last token left, for a layer that
     mixes every token with the one before it)."""
     arrays: Tuple[PagedArray, ...]
     window: Optional[int] = None
     fixed: Optional["FixedSpec"] = None
+    chunk: Optional[int] = None
 
     def __post_init__(self):
+        if self.chunk is not None and (self.window is not None or self.chunk < 1):
+            raise ValueError("a paged spec keeps a window or the query's own chunk (of at least one position), not both")
         names = [a.name for a in self.arrays]
         if len(set(names)) != len(names):
             raise ValueError(f"a paged spec names an array twice: {names}")
@@ -133,13 +138,13 @@ class PagedSpec:
 
 
 def kv_spec(kv_heads: int, head_dim: int, window: Optional[int] = None, v_transposed: bool = False,
-            value_dim: Optional[int] = None) -> PagedSpec:
+            value_dim: Optional[int] = None, chunk: Optional[int] = None) -> PagedSpec:
     """Keys and values of grouped-query attention: K [kv_heads, page, head_dim]
     and V the same (value_dim wide where values have a size of their own), or
     transposed inside the page [kv_heads, value_dim, page]."""
     value_dim = head_dim if value_dim is None else value_dim
     v_shape = (kv_heads, value_dim, PAGE) if v_transposed else (kv_heads, PAGE, value_dim)
-    return PagedSpec((PagedArray("k", (kv_heads, PAGE, head_dim)), PagedArray("v", v_shape)), window)
+    return PagedSpec((PagedArray("k", (kv_heads, PAGE, head_dim)), PagedArray("v", v_shape)), window, chunk=chunk)
 
 
 @dataclass(frozen=True)
@@ -201,7 +206,7 @@ def with_fixed_arrays(spec: StateSpec, arrays: Sequence[FixedArray]) -> StateSpe
     old = fixed_part(spec)
     both = FixedSpec(arrays=(old.all_arrays() if old is not None else ()) + arrays)
     if isinstance(spec, PagedSpec):
-        return PagedSpec(spec.arrays, spec.window, both)
+        return PagedSpec(spec.arrays, spec.window, both, spec.chunk)
     return both
 
 
@@ -315,7 +320,7 @@ class CacheManager:
         sizes = [int(n_pages)] * len(specs) if isinstance(n_pages, int) else [int(n) for n in n_pages]
         if len(sizes) != len(specs):
             raise ValueError(f"{len(sizes)} pool sizes were given for {len(specs)} groups")
-        windows = (ctypes.c_int32 * max(1, len(specs)))(*[s.window or 0 for s in specs])
+        windows = (ctypes.c_int32 * max(1, len(specs)))(*[-s.chunk if s.chunk else (s.window or 0) for s in specs])
         pool_sizes = (ctypes.c_int32 * max(1, len(specs)))(*sizes)
         self._c = self._lib.imparo_cache_new(len(specs), windows, page_size, pool_sizes, n_slots)
         if not self._c:

@@ -18,3 +18,7 @@ from . import kosalorn as _kosalorn
 from .kosalorn import KosalornConfig
 
 register_architecture(_kosalorn.ARCHITECTURE, KosalornConfig.from_dict, _kosalorn.build_plan)
+from . import mepapel as _mepapel
+from .mepapel import MepapelConfig
+
+register_architecture(_mepapel.ARCHITECTURE, MepapelConfig.from_dict, _mepapel.build_plan)

@@ -73,7 +73,8 @@ int imparo_qk_norm_rope_store(const float* qkv, const float* q_weight, const flo
                               int v_transposed, imparo_stream stream);
 
 // Causal grouped-query attention over the paged cache; one query per (token,
-// head); keys lo..pos with lo = max(0, pos + 1 - window) (window 0: all keys).
+// head); keys lo..pos with lo = max(0, pos + 1 - window) (window 0: all keys; window < 0: the keys of the query's
+// own chunk, lo = pos - pos % -window; the matrix-core attention kernels below read `window` the same way).
 int imparo_attention(const void* q, const void* k_cache, const void* v_cache, void* out, int dtype,
                      const int32_t* positions, const int32_t* row_of_token,
                      const int32_t* block_table, int table_stride, int page_size,
@@ -171,6 +172,43 @@ int imparo_hgrn2_scan(const float* rows, int ld, int q_off, int f_off, int v_off
                       int heads, int dim, int vdim, int chunk_tokens, int max_chunks, float* chunk_state,
                       float* chunk_decay, imparo_stream stream);
 
+// ---- recurrences with a matrix of state a head and one decay a head and token
+// Per request (row), head and token in order:  S <- a S + k v^T, out = S^T q;  with `beta` the gated delta rule
+// S <- a S, u = sigmoid(beta) (v - S^T k), S <- S + k u^T, out = S^T q. q, k, v are float32 rows (a token's row ld
+// floats apart, heads from off on; head h reads q head h / q_div and k head h / k_div). a = decay_const[h], or
+// exp(-rate[h] softplus(step[t, h] + step_bias[h])); with v_times_step v is multiplied by that softplus; with
+// `skip`, out += skip[h] v (v as it came). state [slots, heads, dim, vdim] float32; out [tokens, heads * vdim]
+// float32. dim <= 512. chunk_tokens 0: one launch. Otherwise (a multiple of 8, not with beta) segments are walked
+// in chunks side by side, in three launches; max_chunks >= ceil(longest segment / chunk_tokens); chunk_state
+// [n_rows * max_chunks, heads, dim, vdim] and chunk_decay [n_rows * max_chunks, heads] float32 are scratch.
+int imparo_decay_scan(const float* q, int q_ld, int q_off, int q_div, const float* k, int k_ld, int k_off, int k_div,
+                      const float* v, int v_ld, int v_off, const float* decay_const, const float* step, int step_ld,
+                      int step_off, const float* step_bias, const float* rate, int v_times_step, const float* beta,
+                      int beta_ld, int beta_off, const float* skip, float* state, const int32_t* seg_start,
+                      const int32_t* seg_len, const int32_t* slot, float* out, int n_rows, int heads, int dim, int vdim,
+                      int chunk_tokens, int max_chunks, float* chunk_state, float* chunk_decay, imparo_stream stream);
+// Heads of `dim` columns from `off` on in float32 rows, in place: divided by sqrt(sum of squares + unit_eps) if
+// `unit`, the first 2 n_freq dimensions rotated by position (pairs (i, i + n_freq), or neighbours if interleaved),
+// multiplied by scale_first (heads below n_first) or scale_rest.
+int imparo_head_prepare(float* rows, int ld, int off, int n_tokens, int heads, int dim, int unit, float unit_eps,
+                        const float* inv_freq, int n_freq, int interleaved, const int32_t* positions, int n_first,
+                        float scale_first, float scale_rest, imparo_stream stream);
+// A row of `width` float32 values in `groups` equal parts, with g = silu(gate[t, gate_off + c]) (gate null: 1):
+// gate_first: (x g) / rms_part(x g) * w; otherwise x / rms_part(x) * w * g (w null: 1).
+int imparo_gated_group_norm(const float* x, const float* gate, int gate_ld, int gate_off, const float* w, void* out,
+                            int out_dtype, int n_tokens, int width, int groups, float eps, int gate_first,
+                            imparo_stream stream);
+// out[t, j] = g sigmoid(alpha g) (u + 1), g = min(gu[t, j], limit), u = clamp(gu[t, hidden + j], -limit, limit);
+// columns from `hidden` to out_ld are zero.
+int imparo_clamped_glu(const float* gu, void* out, int out_dtype, int n_tokens, int hidden, int out_ld, float limit,
+                       float alpha, imparo_stream stream);
+// out[t] = factor (rms_norm(a[t]) wa + rms_norm(b[t]) wb); a and b float32 [slices, tokens, width], added in order.
+int imparo_normed_sum(const float* a, int a_slices, const float* wa, const float* b, int b_slices, const float* wb,
+                      float* out, int n_tokens, int width, float eps, float factor, imparo_stream stream);
+// out[t] += sigmoid(z[t, z_col]) * (the sum of y's slices)[t].
+int imparo_gated_row_add(float* out, const float* y, int y_slices, const float* z, int z_ld, int z_col, int n_tokens,
+                         int width, imparo_stream stream);
+
 // ---- pieces of a parallel block with gated sublayers
 // x += a * sigmoid(gates[:, :width]) (+ b * sigmoid(gates[:, width : 2 width]), b may be null); with `copy`
 // the new x is also stored there in copy_dtype. x float32 [tokens, width]; a and b float32 [slices, tokens, width],
@@ -182,6 +220,9 @@ int imparo_side_gate(const float* z, const void* table, int table_dtype, int tab
                      int vocab, void* out, int out_dtype, int n_tokens, int dim, int out_ld, imparo_stream stream);
 // x[i] += y[i] for i < n.
 int imparo_add_rows(float* x, const float* y, long long n, imparo_stream stream);
+// out[i] = x[rows ? rows[i] : i] in out_dtype: float32 rows as a product reads them (rows null: all n_out rows).
+int imparo_cast_rows(const float* x, const int32_t* rows, void* out, int out_dtype, int n_out, int width,
+                     imparo_stream stream);
 
 // Matrix-core attention, bfloat16, V cache transposed, page_size a power of two
 // >= 16, head_dim a multiple of 16 up to 128.
@@ -499,8 +540,13 @@ int imparo_embed_gather_scaled(const void* table, int table_dtype, const int32_t
 // route: scores = softmax(logits[t, :n_router]) (scoring 0) or the sigmoid of each output (scoring 1); the `top`
 // largest of score + correction are chosen (of equal ones the lowest index), choice [tokens, top] holds their
 // indices and weight [tokens, top] their scores.
+// Beyond that: a token's logits lie logits_ld floats apart (at least n_router); with groups > 1 (at most 64) the
+// outputs form that many equal groups of neighbours, a group's score is the sum of its two largest choice scores
+// (score + correction) and only outputs of the `keep` best groups can be chosen; with `normalize` the chosen scores
+// are divided by their sum + 1e-20; the weights are multiplied by `scale` at the end.
 int imparo_moe_route(const float* logits, const float* correction, int32_t* choice, float* weight,
-                     int n_tokens, int n_router, int top, int scoring, imparo_stream stream);
+                     int n_tokens, int n_router, int top, int scoring, int logits_ld, int groups, int keep,
+                     int normalize, float scale, imparo_stream stream);
 // hidden[slot, j] = silu(w g) * (w u), g = gu[slot, j], u = gu[slot, half + j], w = weight[entry_of_slot[slot]]
 // (weight null: 1): the hidden values of gated experts without biases that read w times their input, from the
 // stacked gate and up products of the input itself. gu float32 [n_slots, 2 half].
@@ -531,7 +577,7 @@ int imparo_moe_route_plan_tokens(void);
 int imparo_moe_route_plan(const float* logits, const float* correction, int32_t* choice, float* weight,
                           int n_tokens, int n_router, int top, int scoring, int n_experts, int tile_rows,
                           int32_t* slot_of_entry, int32_t* entry_of_slot, int32_t* tiles, int max_tiles,
-                          imparo_stream stream);
+                          int logits_ld, int groups, int keep, int normalize, float scale, imparo_stream stream);
 
 // A norm on what a sublayer returns, its add into the stream, and the next norm, in one launch:
 // x[r] += rms_norm(sum of delta's slices [n_delta, n_rows_x, width])[r] * w_post; with w_next,

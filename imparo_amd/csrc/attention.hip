@@ -72,7 +72,7 @@ __global__ void k_attention_wave(const T* __restrict__ q, const T* __restrict__ 
     const int h = (int)(id - (long long)t * heads);
     const int kvh = h / (heads / kv_heads);
     const int pos = positions[t];
-    const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
+    const int lo = first_seen(pos, window);
     const int32_t* table = block_table + (size_t)row_of_token[t] * table_stride;
 
     float* qr = q_rows[wave];
@@ -145,7 +145,7 @@ static int check_attention_args(const void* q, const void* k_cache, const void* 
     if (!q || !k_cache || !v_cache || !out || !positions || !row_of_token || !block_table) return IMPARO_BAD_ARGUMENT;
     if (n_tokens < 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0) return IMPARO_BAD_ARGUMENT;
     if (head_dim <= 0 || head_dim > ATT_MAX_HEAD_DIM) return IMPARO_BAD_ARGUMENT;
-    if (page_size <= 0 || table_stride <= 0 || n_pages <= 0 || window < 0) return IMPARO_BAD_ARGUMENT;
+    if (page_size <= 0 || table_stride <= 0 || n_pages <= 0) return IMPARO_BAD_ARGUMENT;
     return IMPARO_OK;
 }
 

@@ -305,7 +305,7 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 4 : 2) void k_attn_decod
     const int row = rows[ri];
     const int t = seg_start[row];
     const int pos = positions[t];
-    const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
+    const int lo = first_seen(pos, window);
     const int last = FROM_QKV ? pos - 1 : pos;              // the last key that is in the cache
     const int k_begin = max(split * DEC_SPLIT, lo & ~31);
     const int k_end = min((split + 1) * DEC_SPLIT, last + 1);
@@ -477,7 +477,7 @@ __global__ void k_attn_decode_merge(const float* __restrict__ part_o, const floa
     const bool works = sub < side;
     const int t = seg_start[rows[ri]];
     const int pos = positions[t];
-    const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
+    const int lo = first_seen(pos, window);
     const int s_lo = (lo & ~15) / DEC_SPLIT, s_hi = pos / DEC_SPLIT;
     const size_t base = ((size_t)ri * heads + head) * n_splits;
     float ms = -INFINITY;
@@ -597,7 +597,7 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
     // the block's key range: from the lowest key its first query may read to its last query's position
     const int blk_first = pos0 + tile * 64;
     const int blk_last = pos0 + min(len, tile * 64 + 64) - 1;
-    const int blk_lo = window > 0 ? max(0, blk_first + 1 - window) : 0;
+    const int blk_lo = first_seen(blk_first, window);
 
     // this wave's queries
     const int q_first = tile * 64 + wave * 16;
@@ -607,10 +607,10 @@ __global__ __launch_bounds__(MFMA_WAVES * 64) void k_attn_prefill(
     const int pos_q = pos0 + qi;
     const int pos_first = pos0 + q_first;
     const int pos_last = pos0 + min(len, q_first + 16) - 1;
-    const int lo_q = window > 0 ? max(0, pos_q + 1 - window) : 0;
+    const int lo_q = first_seen(pos_q, window);
     const int hi_q = qvalid ? pos_q : -1;
-    const int lo_all = window > 0 ? max(0, pos_first + 1 - window) : 0;
-    const int lo_max = window > 0 ? max(0, pos_last + 1 - window) : 0;
+    const int lo_all = first_seen(pos_first, window);
+    const int lo_max = first_seen(pos_last, window);
     WaveState<ND> st;
     load_q<ND>(st, q + ((size_t)(t0 + min(qi, len - 1)) * heads + head) * D, qvalid && wave_on, lane);
     const float scale_log2 = scale * 1.44269504088896340736f;
@@ -837,7 +837,7 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
     // of keys and leaves (max, sum, unnormalised output) per query for the merge kernel
     const int blk_first = pos0 + tile * qt;
     int blk_last = pos0 + min(len, tile * qt + qt) - 1;
-    int blk_lo = window > 0 ? max(0, blk_first + 1 - window) : 0;
+    int blk_lo = first_seen(blk_first, window);
     const int n_splits = (int)gridDim.z, split = (int)blockIdx.z;
     if (n_splits > 1) {
         const int first_tile = blk_lo / PX_KEYS, tiles_all = blk_last / PX_KEYS - first_tile + 1;
@@ -853,8 +853,8 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
     const bool wave_on = q_first < len;
     const int pos_first = pos0 + q_first;
     const int pos_last = pos0 + min(len, q_first + QW) - 1;
-    const int lo_all = window > 0 ? max(0, pos_first + 1 - window) : 0;
-    const int lo_max = window > 0 ? max(0, pos_last + 1 - window) : 0;
+    const int lo_all = first_seen(pos_first, window);
+    const int lo_max = first_seen(pos_last, window);
     int lo_q[HALVES], hi_q[HALVES];
     bool qvalid[HALVES];
     Frag8 qf[HALVES][NK];
@@ -872,7 +872,7 @@ __global__ __launch_bounds__(MFMA_WAVES * 64, ND <= 4 ? 2 : 1) void k_attn_prefi
         const int qi = q_first + 16 * h + c;
         qvalid[h] = qi < len;
         const int pos_q = pos0 + qi;
-        lo_q[h] = max(window > 0 ? max(0, pos_q + 1 - window) : 0, blk_lo);
+        lo_q[h] = max(first_seen(pos_q, window), blk_lo);
         hi_q[h] = (qvalid[h] && has_keys) ? min(pos_q, blk_last) : -1;
         const bf16_t* qrow = q + ((size_t)(t0 + min(qi, len - 1)) * heads + head) * D + 8 * g;
 #pragma unroll
@@ -1229,7 +1229,7 @@ static int check_common(const void* q, const void* k_cache, const void* v_cache,
     if (heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0) return IMPARO_BAD_ARGUMENT;
     if (head_dim <= 0 || head_dim % 16 != 0 || head_dim > 128) return IMPARO_BAD_ARGUMENT;
     if (page_size < 16 || (page_size & (page_size - 1)) != 0) return IMPARO_BAD_ARGUMENT;
-    if (table_stride <= 0 || n_pages <= 0 || window < 0) return IMPARO_BAD_ARGUMENT;
+    if (table_stride <= 0 || n_pages <= 0) return IMPARO_BAD_ARGUMENT;
     return IMPARO_OK;
 }
 

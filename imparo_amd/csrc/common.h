@@ -101,6 +101,12 @@ __device__ __forceinline__ void rotation_of(int pos, float inv_freq, float& sn, 
     if (quarter == 1 || quarter == 2) cs = -cs;
     if (quarter >= 2) sn = -sn;
 }
+// The first position a query at `pos` sees. window > 0: the last `window` positions up to its own; window < 0:
+// the positions of its own chunk, chunks of -window positions counted from position 0; 0: every position
+// before it. Never decreases with pos, which is all the attention kernels ask of it.
+__device__ __forceinline__ int first_seen(int pos, int window) {
+    return window > 0 ? max(0, pos + 1 - window) : window < 0 ? pos - pos % (-window) : 0;
+}
 __device__ __forceinline__ float head_norm_scale(float sum_squares, int head_dim, float eps) {
     return 1.0f / sqrtf(sum_squares / (float)head_dim + eps);
 }
@@ -116,6 +122,7 @@ __device__ __forceinline__ void wave_lds_sync() {
 // One per file of kernels: loads that file's code onto the current device (imparo_load_code calls them all).
 int imparo_load_code_attention();
 int imparo_load_code_attention_mfma();
+int imparo_load_code_decay_scan();
 int imparo_load_code_decode_rows();
 int imparo_load_code_diff_attention();
 int imparo_load_code_elementwise();

@@ -1,0 +1,464 @@
+// Recurrences with a matrix of state a head and one decay a head and token:
+//   S <- a S + k v^T,                 o = S^T q                  (a linear attention with decay)
+//   S <- a S;  u = b (v - S^T k);  S <- S + k u^T,  o = S^T q    (the gated delta rule)
+// S [dim, vdim] float32 per request and head, carried from token to token. The decay a is a constant of
+// the head, or exp(-rate_h softplus(raw + bias_h)) of a projected number (the step; the values may be
+// multiplied by that step, as a state-space layer does, and the head's result may take D_h x on top). b is
+// the sigmoid of a projected number. Heads may share queries and keys in groups of neighbours (q_div, k_div
+// heads read one). Decays, steps, gates, the state and every sum are float32 whatever the engine's dtype.
+//
+// A block takes one request's segment, one head and a run of value columns. A thread keeps a slice of one
+// column of S in registers: KS neighbouring lanes share a column, so that the sums over dim (the delta
+// rule's S^T k, every o) end with a few exchanges inside a wave. The tokens' q, k, v and scalars come
+// through LDS eight tokens at a time. Every sum runs in an order that dim alone decides.
+//
+// A long segment of the first form is walked in three launches, its chunks side by side (the recurrence
+// is linear in S with a scalar factor: after a chunk S = (product of the chunk's a) S_before + what the chunk
+// makes of a zero state). The delta rule's transition is a matrix (a (I - b k k^T)), so it is walked in one.
+//
+// Beside it: what such mixers do to a head before the walk (unit length, rotation, a factor) and to the
+// heads behind it (a gate and a norm in groups of the row).
+#include "common.h"
+#include "api.h"
+
+#define DS_KPT 16             // entries of a column a thread keeps at most
+#define DS_TOKENS 8           // tokens staged in LDS at once
+#define DS_MAX_THREADS 256
+#define DS_MAX_DIM 512
+
+__device__ __forceinline__ float ds_sigmoid(float z) { return 1.0f / (1.0f + expf(-z)); }
+__device__ __forceinline__ float ds_silu(float z) { return z / (1.0f + expf(-z)); }
+__device__ __forceinline__ float ds_softplus(float z) { return z > 20.0f ? z : log1pf(expf(z)); }
+
+struct DecayScanArgs {
+    const float* q; int q_ld, q_off, q_div;      // head h reads q head h / q_div
+    const float* k; int k_ld, k_off, k_div;
+    const float* v; int v_ld, v_off;
+    const float* decay_const;                    // [heads], or null: the decay comes from `step`
+    const float* step; int step_ld, step_off;    // raw steps [tokens, heads]
+    const float* step_bias;                      // [heads]
+    const float* rate;                           // [heads]: a = exp(-rate softplus(raw + bias))
+    int v_times_step;                            // v <- softplus(raw + bias) v
+    const float* beta; int beta_ld, beta_off;    // raw [tokens, heads], the delta rule's only
+    const float* skip;                           // [heads] or null: o += skip_h v (v as it came)
+    float* state;                                // [slots, heads, dim, vdim]
+    const int32_t* seg_start; const int32_t* seg_len; const int32_t* slot;
+    float* out;                                  // [tokens, heads * vdim]
+    int heads, dim, vdim, kpt;
+    int chunk_tokens, max_chunks;
+    float* chunk_state;                          // [rows * max_chunks, heads, dim, vdim]
+    float* chunk_decay;                          // [rows * max_chunks, heads]
+};
+
+// MODE 0: a segment from its request's state to its end. With chunks (blockIdx.x = row * max_chunks + chunk):
+// MODE 1: a chunk that is not the segment's last, from a zero state: its end state goes to chunk_state, the
+// product of its decays to chunk_decay, no results; MODE 2: a chunk from the state chunk_state holds for it,
+// with results; the last chunk writes the request's state.
+template <int KS, int MODE, bool DELTA>
+__global__ __launch_bounds__(DS_MAX_THREADS) void k_decay_scan(const DecayScanArgs A) {
+    __shared__ float sq[DS_TOKENS][DS_MAX_DIM], sk[DS_TOKENS][DS_MAX_DIM], sv[DS_TOKENS][DS_MAX_THREADS];
+    __shared__ float sa[DS_TOKENS], sb[DS_TOKENS], sdt[DS_TOKENS];
+    const int VB = blockDim.x / KS;                      // value columns of a block
+    const int r = MODE == 0 ? blockIdx.x : blockIdx.x / A.max_chunks;
+    const int chunk = MODE == 0 ? 0 : blockIdx.x - r * A.max_chunks;
+    const int h = blockIdx.y, v0 = blockIdx.z * VB;
+    const int tid = threadIdx.x, ks = tid % KS, vl = tid / KS;
+    const int v = v0 + vl;
+    const int heads = A.heads, dim = A.dim, vdim = A.vdim, kpt = A.kpt;
+    const bool live = v < vdim;
+    const int n_all = A.seg_len[r];
+    const int n_chunks = MODE == 0 ? 1 : (n_all + A.chunk_tokens - 1) / A.chunk_tokens;
+    if (MODE == 1 && chunk >= n_chunks - 1) return;      // (the whole block)
+    if (MODE == 2 && chunk >= n_chunks) return;
+    const int first = A.seg_start[r] + (MODE == 0 ? 0 : chunk * A.chunk_tokens);
+    const int n = MODE == 0 ? n_all : min(A.chunk_tokens, n_all - chunk * A.chunk_tokens);
+    const int dkp = KS * kpt;                            // dim, filled up to whole slices
+    const int qh = h / A.q_div, kh = h / A.k_div;
+    float* S_at = A.state + (((size_t)A.slot[r] * heads + h) * dim) * vdim;
+    float* C_at = MODE == 0 ? nullptr : A.chunk_state + (((size_t)blockIdx.x * heads + h) * dim) * vdim;
+    float S[DS_KPT];
+    float decay_all = 1.f;
+#pragma unroll
+    for (int j = 0; j < DS_KPT; ++j) {
+        const int k = ks * kpt + j;
+        if constexpr (MODE == 1)
+            S[j] = 0.f;
+        else
+            S[j] = (j < kpt && k < dim && live) ? (MODE == 0 ? S_at : C_at)[(size_t)k * vdim + v] : 0.f;
+    }
+    const float skip = A.skip ? A.skip[h] : 0.f;
+    for (int t0 = 0; t0 < n; t0 += DS_TOKENS) {
+        const int nt = min(DS_TOKENS, n - t0);
+        __syncthreads();                                 // the last batch has been read
+        for (int i = tid; i < nt * dkp; i += blockDim.x) {
+            const int tok = i / dkp, k = i - tok * dkp;
+            const size_t t = (size_t)(first + t0 + tok);
+            sq[tok][k] = k < dim ? A.q[t * A.q_ld + A.q_off + qh * dim + k] : 0.f;   // beyond dim: a state that stays zero
+            sk[tok][k] = k < dim ? A.k[t * A.k_ld + A.k_off + kh * dim + k] : 0.f;
+        }
+        for (int i = tid; i < nt * VB; i += blockDim.x) {
+            const int tok = i / VB, c = i - tok * VB;
+            sv[tok][c] = (v0 + c) < vdim ? A.v[(size_t)(first + t0 + tok) * A.v_ld + A.v_off + h * vdim + v0 + c] : 0.f;
+        }
+        if (tid < nt) {
+            const size_t t = (size_t)(first + t0 + tid);
+            float a, dt = 1.f;
+            if (A.decay_const) {
+                a = A.decay_const[h];
+            } else {
+                dt = ds_softplus(A.step[t * A.step_ld + A.step_off + h] + A.step_bias[h]);
+                a = expf(-A.rate[h] * dt);
+            }
+            sa[tid] = a;
+            sdt[tid] = A.v_times_step ? dt : 1.f;
+            sb[tid] = DELTA ? ds_sigmoid(A.beta[t * A.beta_ld + A.beta_off + h]) : 1.f;
+        }
+        __syncthreads();
+        for (int tok = 0; tok < nt; ++tok) {
+            const float a = sa[tok];
+            const float raw = sv[tok][vl];
+            float val = raw * sdt[tok];
+            float acc = 0.f;
+            if constexpr (DELTA) {
+                float seen = 0.f;
+#pragma unroll
+                for (int j = 0; j < DS_KPT; ++j)
+                    if (j < kpt) {
+                        S[j] *= a;
+                        seen = fmaf(S[j], sk[tok][ks * kpt + j], seen);
+                    }
+#pragma unroll
+                for (int off = 1; off < KS; off <<= 1) seen += __shfl_xor(seen, off, WAVE);
+                val = sb[tok] * (val - seen);
+#pragma unroll
+                for (int j = 0; j < DS_KPT; ++j)
+                    if (j < kpt) {
+                        S[j] = fmaf(sk[tok][ks * kpt + j], val, S[j]);
+                        acc = fmaf(S[j], sq[tok][ks * kpt + j], acc);
+                    }
+            } else {
+#pragma unroll
+                for (int j = 0; j < DS_KPT; ++j)
+                    if (j < kpt) {
+                        S[j] = fmaf(sk[tok][ks * kpt + j], val, a * S[j]);
+                        if constexpr (MODE != 1) acc = fmaf(S[j], sq[tok][ks * kpt + j], acc);
+                    }
+                if constexpr (MODE == 1) decay_all *= a;
+            }
+            if (MODE != 1) {
+#pragma unroll
+                for (int off = 1; off < KS; off <<= 1) acc += __shfl_xor(acc, off, WAVE);
+                if (ks == 0 && live)
+                    A.out[(size_t)(first + t0 + tok) * heads * vdim + (size_t)h * vdim + v] = fmaf(skip, raw, acc);
+            }
+        }
+    }
+    if (MODE == 2 && chunk != n_chunks - 1) return;
+    float* end_at = MODE == 1 ? C_at : S_at;
+#pragma unroll
+    for (int j = 0; j < DS_KPT; ++j) {
+        const int k = ks * kpt + j;
+        if (j < kpt && k < dim && live) end_at[(size_t)k * vdim + v] = S[j];
+    }
+    if (MODE == 1 && tid == 0 && blockIdx.z == 0) A.chunk_decay[(size_t)blockIdx.x * heads + h] = decay_all;
+}
+
+// One thread a state entry: the request's state walks over the chunks' ends; chunk_state[chunk] turns from
+// "what the chunk makes of a zero state" into "the state the chunk starts from".
+__global__ void k_decay_carry(float* __restrict__ chunk_state, const float* __restrict__ chunk_decay,
+                              const float* __restrict__ state, const int32_t* __restrict__ seg_len,
+                              const int32_t* __restrict__ slot, int n_rows, int heads, int dim, int vdim,
+                              int chunk_tokens, int max_chunks) {
+    const long long per_head = (long long)dim * vdim, per_row = per_head * heads;
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_rows * per_row) return;
+    const int r = (int)(i / per_row);
+    const long long e = i - r * per_row;
+    const int h = (int)(e / per_head);
+    const int n_chunks = (seg_len[r] + chunk_tokens - 1) / chunk_tokens;
+    float S = state[(size_t)slot[r] * per_row + e];
+    for (int c = 0; c < n_chunks; ++c) {
+        float* at = chunk_state + ((size_t)r * max_chunks + c) * per_row + e;
+        const bool more = c < n_chunks - 1;
+        const float made = more ? *at : 0.f;
+        *at = S;
+        if (more) S = fmaf(chunk_decay[((size_t)r * max_chunks + c) * heads + h], S, made);
+    }
+}
+
+extern "C" int imparo_decay_scan(const float* q, int q_ld, int q_off, int q_div, const float* k, int k_ld, int k_off,
+                                 int k_div, const float* v, int v_ld, int v_off, const float* decay_const,
+                                 const float* step, int step_ld, int step_off, const float* step_bias,
+                                 const float* rate, int v_times_step, const float* beta, int beta_ld, int beta_off,
+                                 const float* skip, float* state, const int32_t* seg_start, const int32_t* seg_len,
+                                 const int32_t* slot, float* out, int n_rows, int heads, int dim, int vdim,
+                                 int chunk_tokens, int max_chunks, float* chunk_state, float* chunk_decay,
+                                 imparo_stream stream) {
+    if (!q || !k || !v || !state || !seg_start || !seg_len || !slot || !out) return IMPARO_BAD_ARGUMENT;
+    if (!decay_const && (!step || !step_bias || !rate)) return IMPARO_BAD_ARGUMENT;
+    if (v_times_step && decay_const) return IMPARO_BAD_ARGUMENT;
+    if (chunk_tokens < 0 || chunk_tokens % DS_TOKENS) return IMPARO_BAD_ARGUMENT;
+    if (chunk_tokens && (beta || max_chunks < 1 || !chunk_state || !chunk_decay)) return IMPARO_BAD_ARGUMENT;
+    if (n_rows < 0 || heads < 1 || dim < 1 || dim > DS_MAX_DIM || vdim < 1) return IMPARO_BAD_ARGUMENT;
+    if (q_div < 1 || k_div < 1 || heads % q_div || heads % k_div) return IMPARO_BAD_ARGUMENT;
+    if (q_off < 0 || k_off < 0 || v_off < 0 || q_ld < q_off + heads / q_div * dim || k_ld < k_off + heads / k_div * dim ||
+        v_ld < v_off + heads * vdim)
+        return IMPARO_BAD_ARGUMENT;
+    if (step && (step_off < 0 || step_ld < step_off + heads)) return IMPARO_BAD_ARGUMENT;
+    if (beta && (beta_off < 0 || beta_ld < beta_off + heads)) return IMPARO_BAD_ARGUMENT;
+    if (n_rows == 0) return IMPARO_OK;
+    int ks = 1;
+    while ((dim + ks - 1) / ks > DS_KPT) ks *= 2;
+    const int kpt = (dim + ks - 1) / ks;
+    hipStream_t s = (hipStream_t)stream;
+    // a block is as many value columns as fill it, in whole waves
+    int threads = (ks * vdim + WAVE - 1) / WAVE * WAVE;
+    threads = threads > DS_MAX_THREADS ? DS_MAX_THREADS : threads;
+    const int vb = threads / ks;
+    const int chunks = chunk_tokens ? max_chunks : 1;
+    if ((long long)n_rows * chunks > 0x7fffffffLL) return IMPARO_BAD_ARGUMENT;
+    const dim3 grid(n_rows * chunks, heads, (vdim + vb - 1) / vb);
+    const DecayScanArgs args{q, q_ld, q_off, q_div, k, k_ld, k_off, k_div, v, v_ld, v_off, decay_const,
+                             step, step_ld, step_off, step_bias, rate, v_times_step, beta, beta_ld, beta_off, skip,
+                             state, seg_start, seg_len, slot, out, heads, dim, vdim, kpt,
+                             chunk_tokens, max_chunks, chunk_state, chunk_decay};
+#define DS_LAUNCH(KS)                                                                                                \
+    if (beta) {                                                                                                      \
+        k_decay_scan<KS, 0, true><<<grid, threads, 0, s>>>(args);                                                    \
+    } else if (!chunk_tokens) {                                                                                      \
+        k_decay_scan<KS, 0, false><<<grid, threads, 0, s>>>(args);                                                   \
+    } else {                                                                                                         \
+        k_decay_scan<KS, 1, false><<<grid, threads, 0, s>>>(args);                                                   \
+        const long long entries = (long long)n_rows * heads * dim * vdim;                                            \
+        k_decay_carry<<<(unsigned)((entries + 255) / 256), 256, 0, s>>>(chunk_state, chunk_decay, state, seg_len,    \
+                                                                        slot, n_rows, heads, dim, vdim,              \
+                                                                        chunk_tokens, max_chunks);                   \
+        k_decay_scan<KS, 2, false><<<grid, threads, 0, s>>>(args);                                                   \
+    }
+    switch (ks) {
+        case 1: DS_LAUNCH(1); break;
+        case 2: DS_LAUNCH(2); break;
+        case 4: DS_LAUNCH(4); break;
+        case 8: DS_LAUNCH(8); break;
+        case 16: DS_LAUNCH(16); break;
+        case 32: DS_LAUNCH(32); break;
+        default: return IMPARO_BAD_ARGUMENT;
+    }
+#undef DS_LAUNCH
+    return launch_status();
+}
+
+// ---------------------------------------------------------------- a head before the walk
+// One wave per (token, head) over rows [tokens, ld] float32, in place: head j is the `dim` columns from
+// off + j dim. `unit`: the head is divided by sqrt(sum of its squares + unit_eps). Then the first 2 n_freq
+// dimensions are rotated by position (pairs (i, i + n_freq), or neighbours (2i, 2i + 1)), then the head is
+// multiplied by scale_first (heads below n_first) or scale_rest.
+__global__ void k_head_prepare(float* __restrict__ rows, int ld, int off, int n_tokens, int heads, int dim, int unit,
+                               float unit_eps, const float* __restrict__ inv_freq, int n_freq, int interleaved,
+                               const int32_t* __restrict__ positions, int n_first, float scale_first,
+                               float scale_rest) {
+    const int lane = threadIdx.x & (WAVE - 1);
+    const long long id = (long long)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    if (id >= (long long)n_tokens * heads) return;
+    const int t = (int)(id / heads), j = (int)(id - (long long)t * heads);
+    float* x = rows + (size_t)t * ld + off + (size_t)j * dim;
+    float f = j < n_first ? scale_first : scale_rest;
+    if (unit) {
+        float ss = 0.f;
+        for (int i = lane; i < dim; i += WAVE) ss = fmaf(x[i], x[i], ss);
+        f *= 1.0f / sqrtf(wave_sum(ss) + unit_eps);
+    }
+    const int pos = n_freq ? positions[t] : 0;
+    for (int i = lane; i < n_freq; i += WAVE) {
+        const int ia = interleaved ? 2 * i : i, ib = interleaved ? 2 * i + 1 : i + n_freq;
+        float sn, cs;
+        rotation_of(pos, inv_freq[i], sn, cs);
+        const float a = x[ia], b = x[ib];
+        x[ia] = (a * cs - b * sn) * f;
+        x[ib] = (b * cs + a * sn) * f;
+    }
+    for (int i = 2 * n_freq + lane; i < dim; i += WAVE) x[i] *= f;
+}
+
+extern "C" int imparo_head_prepare(float* rows, int ld, int off, int n_tokens, int heads, int dim, int unit,
+                                   float unit_eps, const float* inv_freq, int n_freq, int interleaved,
+                                   const int32_t* positions, int n_first, float scale_first, float scale_rest,
+                                   imparo_stream stream) {
+    if (!rows || n_tokens < 0 || heads < 1 || dim < 1 || off < 0 || ld < off + heads * dim) return IMPARO_BAD_ARGUMENT;
+    if (n_freq < 0 || 2 * n_freq > dim || (n_freq && (!inv_freq || !positions))) return IMPARO_BAD_ARGUMENT;
+    if (n_tokens == 0) return IMPARO_OK;
+    const long long waves = (long long)n_tokens * heads;
+    k_head_prepare<<<(unsigned)((waves + 3) / 4), 4 * WAVE, 0, (hipStream_t)stream>>>(
+        rows, ld, off, n_tokens, heads, dim, unit, unit_eps, inv_freq, n_freq, interleaved, positions, n_first,
+        scale_first, scale_rest);
+    return launch_status();
+}
+
+// ---------------------------------------------------------------- the heads behind the walk
+// out[t, c] for a row of `width` values in `groups` equal parts: with y = x[t, c] and g = silu(gate[t, c]),
+//   gate_first: (y g) / rms_part(y g) * w[c];   otherwise: y / rms_part(y) * w[c] * g     (w null: 1).
+// A wave takes a part (WHOLE_BLOCK: a block does, for long parts).
+template <typename TOut, bool WHOLE_BLOCK>
+__global__ __launch_bounds__(256) void k_gated_group_norm(const float* __restrict__ x, const float* __restrict__ gate,
+                                                          int gate_ld, int gate_off, const float* __restrict__ w,
+                                                          TOut* __restrict__ out, int n_tokens, int width, int groups,
+                                                          float eps, int gate_first) {
+    __shared__ float scratch[16];
+    const int part = width / groups;
+    long long id;
+    int first, stride;
+    if (WHOLE_BLOCK) {
+        id = blockIdx.x;
+        first = threadIdx.x;
+        stride = blockDim.x;
+    } else {
+        id = (long long)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+        first = threadIdx.x & (WAVE - 1);
+        stride = WAVE;
+        if (id >= (long long)n_tokens * groups) return;
+    }
+    const int t = (int)(id / groups), g = (int)(id - (long long)t * groups);
+    const float* xr = x + (size_t)t * width + (size_t)g * part;
+    const float* gr = gate ? gate + (size_t)t * gate_ld + gate_off + (size_t)g * part : nullptr;
+    float ss = 0.f;
+    for (int i = first; i < part; i += stride) {
+        float y = xr[i];
+        if (gate_first && gr) y *= ds_silu(gr[i]);
+        ss = fmaf(y, y, ss);
+    }
+    ss = WHOLE_BLOCK ? block_sum(ss, scratch) : wave_sum(ss);
+    const float rs = 1.0f / sqrtf(ss / (float)part + eps);
+    for (int i = first; i < part; i += stride) {
+        float y = xr[i];
+        const float gv = gr ? ds_silu(gr[i]) : 1.f;
+        if (gate_first) y *= gv;
+        y = y * rs * (w ? w[(size_t)g * part + i] : 1.f);
+        if (!gate_first) y *= gv;
+        store_f32<TOut>(out, (size_t)t * width + (size_t)g * part + i, y);
+    }
+}
+
+extern "C" int imparo_gated_group_norm(const float* x, const float* gate, int gate_ld, int gate_off, const float* w,
+                                       void* out, int out_dtype, int n_tokens, int width, int groups, float eps,
+                                       int gate_first, imparo_stream stream) {
+    if (!x || !out || n_tokens < 0 || width < 1 || groups < 1 || width % groups) return IMPARO_BAD_ARGUMENT;
+    if (gate && (gate_off < 0 || gate_ld < gate_off + width)) return IMPARO_BAD_ARGUMENT;
+    if (out_dtype != IMPARO_F32 && out_dtype != IMPARO_BF16) return IMPARO_BAD_ARGUMENT;
+    if (n_tokens == 0) return IMPARO_OK;
+    hipStream_t s = (hipStream_t)stream;
+    const long long parts = (long long)n_tokens * groups;
+    if (parts > 0x7fffffffLL) return IMPARO_BAD_ARGUMENT;
+    const bool whole = width / groups > 512;
+#define GGN(T, WHOLE, BLOCKS)                                                                                        \
+    k_gated_group_norm<T, WHOLE><<<(unsigned)(BLOCKS), 256, 0, s>>>(x, gate, gate_ld, gate_off, w, (T*)out, n_tokens, \
+                                                                    width, groups, eps, gate_first)
+    if (out_dtype == IMPARO_BF16) {
+        if (whole) GGN(bf16_t, true, parts); else GGN(bf16_t, false, (parts + 3) / 4);
+    } else {
+        if (whole) GGN(float, true, parts); else GGN(float, false, (parts + 3) / 4);
+    }
+#undef GGN
+    return launch_status();
+}
+
+// ---------------------------------------------------------------- a gated unit with bounds
+// gu [tokens, 2 hidden] float32 holds a token's gate values and, `hidden` further on, its up values:
+// g = min(gate, limit), u = clamp(up, -limit, limit), out = g sigmoid(alpha g) (u + 1).
+template <typename TOut>
+__global__ void k_clamped_glu(const float* __restrict__ gu, TOut* __restrict__ out, long long n, int hidden,
+                              int out_ld, float limit, float alpha) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const long long t = i / out_ld;
+    const int j = (int)(i - t * out_ld);
+    float y = 0.f;                                        // columns past `hidden` fill a row up with zeros
+    if (j < hidden) {
+        const float g = fminf(gu[t * 2 * hidden + j], limit);
+        const float u = fminf(fmaxf(gu[t * 2 * hidden + hidden + j], -limit), limit);
+        y = g * ds_sigmoid(alpha * g) * (u + 1.0f);
+    }
+    store_f32<TOut>(out, (size_t)i, y);
+}
+
+extern "C" int imparo_clamped_glu(const float* gu, void* out, int out_dtype, int n_tokens, int hidden, int out_ld,
+                                  float limit, float alpha, imparo_stream stream) {
+    if (!gu || !out || n_tokens < 0 || hidden < 1 || out_ld < hidden) return IMPARO_BAD_ARGUMENT;
+    if (out_dtype != IMPARO_F32 && out_dtype != IMPARO_BF16) return IMPARO_BAD_ARGUMENT;
+    const long long n = (long long)n_tokens * out_ld;
+    if (n == 0) return IMPARO_OK;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (out_dtype == IMPARO_BF16)
+        k_clamped_glu<bf16_t><<<blocks, 256, 0, (hipStream_t)stream>>>(gu, (bf16_t*)out, n, hidden, out_ld, limit, alpha);
+    else
+        k_clamped_glu<float><<<blocks, 256, 0, (hipStream_t)stream>>>(gu, (float*)out, n, hidden, out_ld, limit, alpha);
+    return launch_status();
+}
+
+// ---------------------------------------------------------------- sums of mixers and of experts
+// out[t, c] (+)= sum_i f_i * rms_norm(a_i[t])[c] * w_i[c] over up to two inputs (each maybe in slices that
+// are added in order first): the results of mixers that run side by side, each normed over the row.
+__global__ __launch_bounds__(256) void k_normed_sum(const float* __restrict__ a, int a_slices, const float* __restrict__ wa,
+                                                    const float* __restrict__ b, int b_slices, const float* __restrict__ wb,
+                                                    float* __restrict__ out, int n_tokens, int width, float eps,
+                                                    float factor) {
+    __shared__ float scratch[16];
+    const int t = blockIdx.x;
+    const size_t stride = (size_t)n_tokens * width;
+    float ssa = 0.f, ssb = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        float ya = 0.f, yb = 0.f;
+        for (int s = 0; s < a_slices; ++s) ya += a[s * stride + (size_t)t * width + i];
+        for (int s = 0; s < b_slices; ++s) yb += b[s * stride + (size_t)t * width + i];
+        ssa = fmaf(ya, ya, ssa);
+        ssb = fmaf(yb, yb, ssb);
+    }
+    const float ra = 1.0f / sqrtf(block_sum(ssa, scratch) / (float)width + eps);
+    const float rb = 1.0f / sqrtf(block_sum(ssb, scratch) / (float)width + eps);
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        float ya = 0.f, yb = 0.f;
+        for (int s = 0; s < a_slices; ++s) ya += a[s * stride + (size_t)t * width + i];
+        for (int s = 0; s < b_slices; ++s) yb += b[s * stride + (size_t)t * width + i];
+        out[(size_t)t * width + i] = factor * (ya * ra * wa[i] + yb * rb * wb[i]);
+    }
+}
+
+extern "C" int imparo_normed_sum(const float* a, int a_slices, const float* wa, const float* b, int b_slices,
+                                 const float* wb, float* out, int n_tokens, int width, float eps, float factor,
+                                 imparo_stream stream) {
+    if (!a || !b || !wa || !wb || !out || a_slices < 1 || b_slices < 1 || n_tokens < 0 || width < 1)
+        return IMPARO_BAD_ARGUMENT;
+    if (n_tokens == 0) return IMPARO_OK;
+    k_normed_sum<<<n_tokens, 256, 0, (hipStream_t)stream>>>(a, a_slices, wa, b, b_slices, wb, out, n_tokens, width, eps,
+                                                            factor);
+    return launch_status();
+}
+
+// out[t, c] += sigmoid(z[t, z_col]) * sum over slices of y[s, t, c]: an expert that every token uses, weighed by
+// one gate a token.
+__global__ void k_gated_row_add(float* __restrict__ out, const float* __restrict__ y, int y_slices,
+                                const float* __restrict__ z, int z_ld, int z_col, int n_tokens, int width) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (long long)n_tokens * width) return;
+    const long long t = i / width;
+    float s = 0.f;
+    for (int k = 0; k < y_slices; ++k) s += y[(size_t)k * n_tokens * width + i];
+    out[i] = fmaf(ds_sigmoid(z[t * z_ld + z_col]), s, out[i]);
+}
+
+extern "C" int imparo_gated_row_add(float* out, const float* y, int y_slices, const float* z, int z_ld, int z_col,
+                                    int n_tokens, int width, imparo_stream stream) {
+    if (!out || !y || !z || y_slices < 1 || z_col < 0 || z_ld <= z_col || n_tokens < 0 || width < 1)
+        return IMPARO_BAD_ARGUMENT;
+    const long long n = (long long)n_tokens * width;
+    if (n == 0) return IMPARO_OK;
+    k_gated_row_add<<<(unsigned)((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(out, y, y_slices, z, z_ld, z_col,
+                                                                                n_tokens, width);
+    return launch_status();
+}
+
+int imparo_load_code_decay_scan() {
+    hipFuncAttributes attributes;
+    return hipFuncGetAttributes(&attributes, reinterpret_cast<const void*>(&k_decay_carry)) == hipSuccess
+               ? IMPARO_OK
+               : IMPARO_LAUNCH_FAILED;
+}

@@ -3,6 +3,7 @@
 //               product that reads the stream itself
 //   side_gate   g[t, j] = gelu_tanh(z[t, j]) * table[token[t], offset + j]
 //   add_rows    x += y
+//   cast_rows   the stream's rows (all, or chosen ones) in another dtype
 // All sums and activations in float32, one order per element whatever the batch.
 #include "common.h"
 #include "api.h"
@@ -101,6 +102,31 @@ extern "C" int imparo_add_rows(float* x, const float* y, long long n, imparo_str
     if (!x || !y || n < 0) return IMPARO_BAD_ARGUMENT;
     if (n == 0) return IMPARO_OK;
     k_add_rows<<<(unsigned)((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(x, y, n);
+    return launch_status();
+}
+
+// out[i] = x[rows ? rows[i] : i] in out's dtype: the stream's rows as a product reads them, without a norm.
+template <typename TOut>
+__global__ void k_cast_rows(const float* __restrict__ x, const int32_t* __restrict__ rows, TOut* __restrict__ out,
+                            int width, long long total) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const long long t = i / width;
+    const long long src = rows ? (long long)rows[t] * width + (i - t * width) : i;
+    store_f32<TOut>(out, (size_t)i, x[src]);
+}
+
+extern "C" int imparo_cast_rows(const float* x, const int32_t* rows, void* out, int out_dtype, int n_out, int width,
+                                imparo_stream stream) {
+    if (!x || !out || n_out < 0 || width < 1) return IMPARO_BAD_ARGUMENT;
+    if (out_dtype != IMPARO_F32 && out_dtype != IMPARO_BF16) return IMPARO_BAD_ARGUMENT;
+    const long long n = (long long)n_out * width;
+    if (n == 0) return IMPARO_OK;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (out_dtype == IMPARO_BF16)
+        k_cast_rows<bf16_t><<<blocks, 256, 0, (hipStream_t)stream>>>(x, rows, (bf16_t*)out, width, n);
+    else
+        k_cast_rows<float><<<blocks, 256, 0, (hipStream_t)stream>>>(x, rows, (float*)out, width, n);
     return launch_status();
 }
 

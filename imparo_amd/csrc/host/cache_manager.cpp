@@ -73,7 +73,7 @@ struct Request {
 
 struct ImparoCache {
     int page_size;
-    std::vector<int> windows;                            // 0 = every position
+    std::vector<int> windows;                            // 0 = every position; w > 0: the last w; w < 0: chunks of -w
     std::vector<ImparoPool> pools;
     ImparoPool slots;
     std::unordered_map<int64_t, Request> live;
@@ -86,8 +86,11 @@ struct ImparoCache {
         }
     }
     int first_needed_page(int g, int next_position) const {
-        if (windows[(size_t)g] <= 0) return 0;
-        return std::max(0, next_position + 1 - windows[(size_t)g]) / page_size;
+        const int w = windows[(size_t)g];
+        if (w == 0) return 0;
+        // a query in a chunk sees its own chunk only: from the chunk's first position
+        if (w < 0) return (next_position - next_position % (-w)) / page_size;
+        return std::max(0, next_position + 1 - w) / page_size;
     }
     void undo(Request& r) {
         for (auto it = r.pending.rbegin(); it != r.pending.rend(); ++it) {
@@ -199,7 +202,7 @@ int imparo_cache_commit(ImparoCache* c, int64_t req, int new_length) {
     r.length = new_length;
     r.pending.clear();
     for (size_t g = 0; g < c->pools.size(); ++g) {
-        if (c->windows[g] <= 0) continue;
+        if (c->windows[g] == 0) continue;
         std::vector<int32_t>& table = r.tables[g];
         const int upto = std::min(c->first_needed_page((int)g, new_length), (int)table.size());
         for (int i = 0; i < upto; ++i)

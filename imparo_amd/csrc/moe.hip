@@ -26,9 +26,19 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 extern "C" int imparo_moe_max_tiles(int n_entries, int n_experts, int tile_rows);
 
 // ---------------------------------------------------------------- route
+// What a router may do beyond scoring and choosing. logits_ld: floats between two tokens' logits (at least
+// n_router; further columns belong to someone else). groups > 1: the router outputs form that many equal
+// groups of neighbours, a group's score is the sum of its two largest choice scores (score + correction), and
+// only outputs of the `keep` best groups can be chosen (of equal groups the lowest). normalize: the chosen
+// scores are divided by their sum + 1e-20. scale: the weights are multiplied by it at the end.
+struct MoeRouteRules {
+    int logits_ld, groups, keep, normalize;
+    float scale;
+};
+
 __device__ __forceinline__ void moe_route_token(const float* __restrict__ logits, const float* __restrict__ correction,
                                                 int32_t* __restrict__ choice, float* __restrict__ weight, int t,
-                                                int n_router, int top, int scoring) {
+                                                int n_router, int top, int scoring, const MoeRouteRules rules) {
     const int lane = threadIdx.x & (WAVE - 1);
     constexpr int PER = MOE_MAX_ROUTER / WAVE;
     float z[PER], pick[PER];
@@ -36,7 +46,7 @@ __device__ __forceinline__ void moe_route_token(const float* __restrict__ logits
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
         const int i = lane + j * WAVE;
-        z[j] = i < n_router ? logits[(size_t)t * n_router + i] : -INFINITY;
+        z[j] = i < n_router ? logits[(size_t)t * rules.logits_ld + i] : -INFINITY;
         m = fmaxf(m, z[j]);
     }
     if (scoring == MOE_SCORE_SIGMOID) {
@@ -61,6 +71,46 @@ __device__ __forceinline__ void moe_route_token(const float* __restrict__ logits
         const int i = lane + j * WAVE;
         pick[j] = i < n_router ? z[j] + (correction ? correction[i] : 0.f) : -INFINITY;
     }
+    if (rules.groups > 1) {
+        // lane g scores group g (at most 64 groups): the sum of its two largest choice scores, read from
+        // the lanes that hold them; then `keep` rounds of a wave-wide argmax mark the groups that stay
+        const int per = n_router / rules.groups;
+        float gscore = -INFINITY;
+        {
+            float b1 = -INFINITY, b2 = -INFINITY;
+            for (int e = 0; e < per; ++e) {
+                // every lane reads output (lane * per + e) of its own group; lanes beyond the groups read output 0
+                const int i = lane < rules.groups ? lane * per + e : 0;
+                float v = -INFINITY;
+#pragma unroll
+                for (int j = 0; j < PER; ++j) {
+                    const float got = __shfl(pick[j], i & (WAVE - 1), WAVE);
+                    if (i / WAVE == j) v = got;
+                }
+                if (v > b1) { b2 = b1; b1 = v; } else if (v > b2) { b2 = v; }
+            }
+            if (lane < rules.groups) gscore = per > 1 ? b1 + b2 : b1;
+        }
+        unsigned long long kept = 0ull;
+        for (int k = 0; k < rules.keep; ++k) {
+            float best = gscore;
+            int at = lane < rules.groups ? lane : 0x7fffffff;
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                const float ob = __shfl_xor(best, off, WAVE);
+                const int oa = __shfl_xor(at, off, WAVE);
+                if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+            }
+            if (at < rules.groups) kept |= 1ull << at;
+            if (lane == at) gscore = -INFINITY;
+        }
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int i = lane + j * WAVE;
+            if (i < n_router && !((kept >> (i / per)) & 1ull)) pick[j] = -INFINITY;
+        }
+    }
+    float chosen_sum = 0.f;
     for (int k = 0; k < top; ++k) {
         // the largest choice score that is left; of equal ones the lowest index
         float best = -INFINITY;
@@ -81,29 +131,44 @@ __device__ __forceinline__ void moe_route_token(const float* __restrict__ logits
         for (int j = 0; j < PER; ++j)
             if (lane + j * WAVE == at) { s = z[j]; pick[j] = -INFINITY; }
         s = wave_sum(s);           // one lane holds it
+        chosen_sum += s;
         if (lane == 0) {
             choice[(size_t)t * top + k] = at;
             weight[(size_t)t * top + k] = s;
         }
     }
+    if (rules.normalize || rules.scale != 1.0f) {
+        const float f = (rules.normalize ? 1.0f / (chosen_sum + 1e-20f) : 1.0f) * rules.scale;
+        if (lane == 0)
+            for (int k = 0; k < top; ++k) weight[(size_t)t * top + k] *= f;
+    }
 }
 
 __global__ void k_moe_route(const float* __restrict__ logits, const float* __restrict__ correction,
                             int32_t* __restrict__ choice, float* __restrict__ weight, int n_tokens, int n_router,
-                            int top, int scoring) {
+                            int top, int scoring, const MoeRouteRules rules) {
     const int t = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
-    if (t < n_tokens) moe_route_token(logits, correction, choice, weight, t, n_router, top, scoring);
+    if (t < n_tokens) moe_route_token(logits, correction, choice, weight, t, n_router, top, scoring, rules);
+}
+
+static bool moe_rules_fit(const MoeRouteRules& r, int n_router, int top) {
+    if (r.logits_ld < n_router || r.groups < 1 || r.groups > WAVE || n_router % r.groups) return false;
+    if (r.groups > 1 && (r.keep < 1 || r.keep > r.groups || r.keep * (n_router / r.groups) < top)) return false;
+    return r.scale == r.scale;
 }
 
 extern "C" int imparo_moe_route(const float* logits, const float* correction, int32_t* choice, float* weight,
-                                int n_tokens, int n_router, int top, int scoring, imparo_stream stream) {
+                                int n_tokens, int n_router, int top, int scoring, int logits_ld, int groups, int keep,
+                                int normalize, float scale, imparo_stream stream) {
     if (!logits || !choice || !weight || n_tokens < 0) return IMPARO_BAD_ARGUMENT;
+    const MoeRouteRules rules{logits_ld, groups, keep, normalize, scale};
+    if (!moe_rules_fit(rules, n_router, top)) return IMPARO_BAD_ARGUMENT;
     if (scoring != MOE_SCORE_SOFTMAX && scoring != MOE_SCORE_SIGMOID) return IMPARO_BAD_ARGUMENT;
     if (n_router < 1 || n_router > MOE_MAX_ROUTER || top < 1 || top > n_router || top > MOE_MAX_TOP)
         return IMPARO_BAD_ARGUMENT;
     if (n_tokens == 0) return IMPARO_OK;
     k_moe_route<<<(n_tokens + 3) / 4, 4 * WAVE, 0, (hipStream_t)stream>>>(logits, correction, choice, weight, n_tokens,
-                                                                         n_router, top, scoring);
+                                                                         n_router, top, scoring, rules);
     return launch_status();
 }
 
@@ -182,13 +247,13 @@ __global__ __launch_bounds__(1024) void k_moe_route_plan(const float* __restrict
                                                          const float* __restrict__ correction,
                                                          int32_t* __restrict__ choice, float* __restrict__ weight,
                                                          int n_tokens, int n_router, int top, int scoring,
-                                                         int n_experts, int tile_rows,
+                                                         const MoeRouteRules rules, int n_experts, int tile_rows,
                                                          int32_t* __restrict__ slot_of_entry,
                                                          int32_t* __restrict__ entry_of_slot,
                                                          int32_t* __restrict__ tiles, int max_tiles) {
     __shared__ MoePlanShared sh;
     for (int t = threadIdx.x / WAVE; t < n_tokens; t += blockDim.x / WAVE)
-        moe_route_token(logits, correction, choice, weight, t, n_router, top, scoring);
+        moe_route_token(logits, correction, choice, weight, t, n_router, top, scoring, rules);
     __threadfence_block();
     __syncthreads();
     moe_plan_block(sh, choice, n_tokens * top, n_experts, tile_rows, slot_of_entry, entry_of_slot, tiles, max_tiles);
@@ -199,8 +264,11 @@ extern "C" int imparo_moe_route_plan_tokens() { return MOE_ROUTE_PLAN_TOKENS; }
 extern "C" int imparo_moe_route_plan(const float* logits, const float* correction, int32_t* choice, float* weight,
                                      int n_tokens, int n_router, int top, int scoring, int n_experts, int tile_rows,
                                      int32_t* slot_of_entry, int32_t* entry_of_slot, int32_t* tiles, int max_tiles,
+                                     int logits_ld, int groups, int keep, int normalize, float scale,
                                      imparo_stream stream) {
     if (!logits || !choice || !weight || !slot_of_entry || !entry_of_slot || !tiles) return IMPARO_BAD_ARGUMENT;
+    const MoeRouteRules rules{logits_ld, groups, keep, normalize, scale};
+    if (!moe_rules_fit(rules, n_router, top)) return IMPARO_BAD_ARGUMENT;
     if (scoring != MOE_SCORE_SOFTMAX && scoring != MOE_SCORE_SIGMOID) return IMPARO_BAD_ARGUMENT;
     if (n_tokens < 0 || n_tokens > MOE_ROUTE_PLAN_TOKENS) return IMPARO_BAD_ARGUMENT;
     if (n_router < 1 || n_router > MOE_MAX_ROUTER || top < 1 || top > n_router || top > MOE_MAX_TOP)
@@ -209,8 +277,8 @@ extern "C" int imparo_moe_route_plan(const float* logits, const float* correctio
     if (max_tiles < imparo_moe_max_tiles(n_tokens * top, n_experts, tile_rows)) return IMPARO_SCRATCH_TOO_SMALL;
     if (n_tokens == 0) return IMPARO_OK;
     k_moe_route_plan<<<1, 1024, 0, (hipStream_t)stream>>>(logits, correction, choice, weight, n_tokens, n_router, top,
-                                                          scoring, n_experts, tile_rows, slot_of_entry, entry_of_slot, tiles,
-                                                          max_tiles);
+                                                          scoring, rules, n_experts, tile_rows, slot_of_entry, entry_of_slot,
+                                                          tiles, max_tiles);
     return launch_status();
 }
 
@@ -714,7 +782,16 @@ __global__ __launch_bounds__(256) void k_post_norm_add(float* __restrict__ x, co
             ss = fmaf(xv[j], xv[j], ss);
         }
     }
-    if (!w_next) return;
+    if (!w_next) {
+        // no norm follows: with an output, the new rows themselves go there in its dtype
+        if (out)
+#pragma unroll
+            for (int j = 0; j < PER; ++j) {
+                const int i = threadIdx.x + j * 256;
+                if (i < width) store_f32<TOut>(out, (size_t)i_out * width + i, xv[j]);
+            }
+        return;
+    }
     const float r2 = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps_next);
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
@@ -734,8 +811,8 @@ static int post_norm_add_launch(float* x, const float* delta, int n_delta, MoeRo
     hipStream_t s = (hipStream_t)stream;
     const size_t stride = (size_t)n_rows_x * width;
     const int write_back = rows ? 0 : 1;
-    const bool to_bf16 = w_next && out_dtype == IMPARO_BF16;
-    if (w_next && out_dtype != IMPARO_BF16 && out_dtype != IMPARO_F32) return IMPARO_BAD_ARGUMENT;
+    const bool to_bf16 = out && out_dtype == IMPARO_BF16;
+    if (out && out_dtype != IMPARO_BF16 && out_dtype != IMPARO_F32) return IMPARO_BAD_ARGUMENT;
 #define POST_NORM(PER)                                                                                              \
     if (to_bf16)                                                                                                    \
         k_post_norm_add<bf16_t, PER><<<n_out, 256, 0, s>>>(x, delta, n_delta, stride, moe, rows, w_post, eps_post,  \

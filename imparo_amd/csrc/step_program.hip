@@ -428,7 +428,7 @@ extern "C" int imparo_load_code() {
                           imparo_load_code_gemm(),      imparo_load_code_rope_cache(),     imparo_load_code_sampling(),
                           imparo_load_code_diff_attention(), imparo_load_code_row_ops(), imparo_load_code_selective_scan(),
                           imparo_load_code_moe(), imparo_load_code_gated_ops(), imparo_load_code_hgrn2(),
-                          imparo_load_code_latent_attention()};
+                          imparo_load_code_latent_attention(), imparo_load_code_decay_scan()};
     for (int s : status)
         if (s != IMPARO_OK) return s;
     return IMPARO_OK;

@@ -70,7 +70,7 @@ _SIGNATURES = {
     "imparo_embed_gather_scaled": [P, I, P, P, I, I, I, F, P],
     "imparo_qk_norm_rope_store_dv": [P, P, P, F, P, I, I, P, P, P, I, I, P, P, P, I, I, I, I, I, I, I, I, I, P],
     "imparo_attention_dv": [P, P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, I, F, I, I, P],
-    "imparo_moe_route": [P, P, P, P, I, I, I, I, P],
+    "imparo_moe_route": [P, P, P, P, I, I, I, I, I, I, I, I, F, P],
     "imparo_moe_gated": [P, P, P, P, I, I, I, P],
     "imparo_attention_latent": [P, P, P, I, P, P, P, I, I, I, I, I, I, I, F, I, P],
     "imparo_latent_store": [P, P, P, F, P, I, I, P, P, P, I, I, I, P, P, P, P, I, I, I, I, I, I, P],
@@ -80,11 +80,22 @@ _SIGNATURES = {
     "imparo_head_gemm": [P, I, I, P, I, P, I, I, I, I, I, I, I, P],
     "imparo_head_gemm_tiles": [P, I, I, P, P, I, I, I, I, I, I, I, P],
     "imparo_hgrn2_scan": [P, I, I, I, I, P, P, P, P, P, P, I, I, I, I, I, I, P, P, P],
+    # q, ld, off, div, k, ld, off, div, v, ld, off, decay_const, step, ld, off, step_bias, rate, v_times_step, beta, ld,
+    # off, skip, state, seg_start, seg_len, slot, out, n_rows, heads, dim, vdim, chunk_tokens, max_chunks, chunk_state,
+    # chunk_decay, stream
+    "imparo_decay_scan": [P, I, I, I, P, I, I, I, P, I, I, P, P, I, I, P, P, I, P, I, I, P, P, P, P, P, P, I, I, I, I, I, I,
+                          P, P, P],
+    "imparo_head_prepare": [P, I, I, I, I, I, I, F, P, I, I, P, I, F, F, P],
+    "imparo_gated_group_norm": [P, P, I, I, P, P, I, I, I, I, F, I, P],
+    "imparo_clamped_glu": [P, P, I, I, I, I, F, F, P],
+    "imparo_normed_sum": [P, I, P, P, I, P, P, I, I, F, F, P],
+    "imparo_gated_row_add": [P, P, I, P, I, I, I, I, P],
     "imparo_gated_sum": [P, P, I, P, I, P, I, P, I, I, I, P],
     "imparo_side_gate": [P, P, I, I, I, P, I, P, I, I, I, I, P],
     "imparo_add_rows": [P, P, c_int64, P],
+    "imparo_cast_rows": [P, P, P, I, I, I, P],
     "imparo_moe_route_plan_tokens": [],
-    "imparo_moe_route_plan": [P, P, P, P, I, I, I, I, I, I, P, P, P, I, P],
+    "imparo_moe_route_plan": [P, P, P, P, I, I, I, I, I, I, P, P, P, I, I, I, I, I, F, P],
     # x, y, h, h_dtype, choice, weight, slot_of_entry, top, n_experts, n_rows_x, rows, w_post, eps_post, w_next, eps_next,
     # out, out_dtype, n_out, width, stream
     "imparo_post_norm_add_moe": [P, P, P, I, P, P, P, I, I, I, P, P, F, P, F, P, I, I, I, P],

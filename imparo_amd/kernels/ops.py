@@ -601,21 +601,22 @@ def poly_norm(z: torch.Tensor, coef: torch.Tensor, eps: float, out: torch.Tensor
 # ------------------------------------------------------------------ selective state-space mixer
 def causal_conv(u: torch.Tensor, channels: int, weight: torch.Tensor, bias: Optional[torch.Tensor],
                 state: Optional[torch.Tensor], row_of_token: torch.Tensor, seg_start: torch.Tensor, seg_len: torch.Tensor,
-                slot: torch.Tensor, out: torch.Tensor, silu: bool = True, single_tokens: bool = False) -> torch.Tensor:
-    """Causal per-channel convolution of each request's segment over the first `channels` columns of u
-    (float32 rows), continued from the request's history, which is advanced: state [slots, taps - 1,
+                slot: torch.Tensor, out: torch.Tensor, silu: bool = True, single_tokens: bool = False,
+                u_off: int = 0) -> torch.Tensor:
+    """Causal per-channel convolution of each request's segment over `channels` columns of u (float32 rows)
+    from column `u_off` on, continued from the request's history, which is advanced: state [slots, taps - 1,
     channels] (None with one tap). The last tap is the current token's."""
     n, u_ld = u.shape
     ch, taps = weight.shape
     n_rows = seg_start.shape[0]
-    if ch != channels or u_ld < channels:
+    if ch != channels or u_off < 0 or u_ld < u_off + channels:
         raise KernelArgumentError(f"causal_conv: a [{ch}, {taps}] filter does not fit {channels} channels of rows of {u_ld}")
     if taps > 1:
         if state is None:
             raise KernelArgumentError("causal_conv: a filter of more than one tap needs a history")
         _dev(state, "conv history", torch.float32, (state.shape[0], taps - 1, channels))
     _check(library().imparo_causal_conv(
-        _dev(u, "conv input", torch.float32), u_ld, _dev(weight, "conv weight", torch.float32),
+        _dev(u, "conv input", torch.float32) + 4 * int(u_off), u_ld, _dev(weight, "conv weight", torch.float32),
         _dev(bias, "conv bias", torch.float32, (channels,)), _dev(state, "conv history", torch.float32) if taps > 1 else 0,
         _dev(row_of_token, "row_of_token", torch.int32, (n,)), _dev(seg_start, "seg_start", torch.int32, (n_rows,)),
         _dev(seg_len, "seg_len", torch.int32, (n_rows,)), _dev(slot, "slot", torch.int32, (n_rows,)),
@@ -758,15 +759,32 @@ MOE_EPILOGUES = {None: 0, "none": 0, "relu2": 1}
 MOE_SCORINGS = {"softmax": 0, "sigmoid": 1}
 
 
+def _route_rules(logits: torch.Tensor, n_router: Optional[int], groups: int, keep: int, normalize: bool, scale: float):
+    """The router outputs among a token's logits and the rules of the choice, as the kernels take them."""
+    r = logits.shape[1] if n_router is None else int(n_router)
+    if not 1 <= r <= logits.shape[1]:
+        raise KernelArgumentError(f"moe_route: {r} router outputs in rows of {logits.shape[1]} logits")
+    groups = int(groups or 1)
+    if groups < 1 or groups > 64 or r % groups or (groups > 1 and not 1 <= keep <= groups):
+        raise KernelArgumentError(f"moe_route: {r} outputs in {groups} groups of which {keep} stay")
+    return r, (logits.shape[1], groups, int(keep or 1), int(bool(normalize)), float(scale))
+
+
 def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], choice: torch.Tensor, weight: torch.Tensor,
-              top: int, scoring: str = "softmax") -> None:
+              top: int, scoring: str = "softmax", n_router: Optional[int] = None, groups: int = 1, keep: int = 1,
+              normalize: bool = False, scale: float = 1.0) -> None:
     """choice[t] = the `top` router outputs with the largest score + correction, weight[t] their scores (as
-    they are); scores are softmax(logits[t]) or, with scoring "sigmoid", the sigmoid of each output."""
-    n, r = logits.shape
+    they are); scores are softmax(logits[t]) or, with scoring "sigmoid", the sigmoid of each output.
+    `n_router`: only the first so many columns of `logits` are router outputs. `groups` > 1: the outputs form
+    that many equal groups of neighbours, a group scores the sum of its two largest score + correction, and
+    only the `keep` best groups' outputs can be chosen. `normalize`: the chosen scores are divided by their
+    sum (+ 1e-20); `scale` multiplies the weights at the end."""
+    n = logits.shape[0]
+    r, rules = _route_rules(logits, n_router, groups, keep, normalize, scale)
     _check(library().imparo_moe_route(
         _dev(logits, "router logits", torch.float32), _dev(correction, "router correction", torch.float32, (r,)),
         _dev(choice, "choice", torch.int32, (n, top)), _dev(weight, "choice weights", torch.float32, (n, top)),
-        n, r, top, MOE_SCORINGS[scoring], _stream()), "moe_route")
+        n, r, top, MOE_SCORINGS[scoring], *rules, _stream()), "moe_route")
 
 
 def moe_gated(gu: torch.Tensor, weight: Optional[torch.Tensor], entry_of_slot: Optional[torch.Tensor],
@@ -793,16 +811,18 @@ def moe_route_plan_tokens() -> int:
 
 def moe_route_plan(logits: torch.Tensor, correction: Optional[torch.Tensor], choice: torch.Tensor, weight: torch.Tensor,
                    top: int, n_experts: int, tile_rows: int, slot_of_entry: torch.Tensor, entry_of_slot: torch.Tensor,
-                   tiles: torch.Tensor, scoring: str = "softmax") -> None:
+                   tiles: torch.Tensor, scoring: str = "softmax", n_router: Optional[int] = None, groups: int = 1,
+                   keep: int = 1, normalize: bool = False, scale: float = 1.0) -> None:
     """`moe_route` and `moe_plan` in one launch, for the few tokens of a decode step."""
-    n, r = logits.shape
+    n = logits.shape[0]
+    r, rules = _route_rules(logits, n_router, groups, keep, normalize, scale)
     _dev(slot_of_entry, "slot_of_entry", torch.int32, (n * top,))
     _dev(entry_of_slot, "entry_of_slot", torch.int32, (n * top,))
     _check(library().imparo_moe_route_plan(
         _dev(logits, "router logits", torch.float32), _dev(correction, "router correction", torch.float32, (r,)),
         _dev(choice, "choice", torch.int32, (n, top)), _dev(weight, "choice weights", torch.float32, (n, top)),
         n, r, top, MOE_SCORINGS[scoring], n_experts, tile_rows, slot_of_entry.data_ptr(), entry_of_slot.data_ptr(),
-        _dev(tiles, "tiles", torch.int32), tiles.shape[0], _stream()), "moe_route_plan")
+        _dev(tiles, "tiles", torch.int32), tiles.shape[0], *rules, _stream()), "moe_route_plan")
 
 
 def moe_tile_rows(n_entries: int, n_experts: int, dtype: torch.dtype) -> int:
@@ -863,7 +883,8 @@ def post_norm_add(x: torch.Tensor, delta, w_post: torch.Tensor, eps_post: float,
                   w_next: Optional[torch.Tensor] = None, eps_next: float = 0.0, out: Optional[torch.Tensor] = None,
                   rows: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """x += rms_norm(delta) * w_post (delta shaped like x, or [slices, *x.shape], added in order); with
-    `w_next`, out = rms_norm(x) * w_next. With `rows` only those rows are taken, into out, and x stays.
+    `w_next`, out = rms_norm(x) * w_next; with `out` and no `w_next`, out = the new x itself in out's dtype.
+    With `rows` only those rows are taken, into out, and x stays.
     `delta` may be what a routed feed-forward left to be combined (an object with y, h, choice, weight,
     slot_of_entry, n_experts): the launch then makes moe_combine's sum itself."""
     n_x, width = x.shape
@@ -872,10 +893,10 @@ def post_norm_add(x: torch.Tensor, delta, w_post: torch.Tensor, eps_post: float,
         top = delta.choice.shape[1]
         if delta.weight is None:
             raise KernelArgumentError("post_norm_add: the experts' sum inside this launch needs the choice's weights")
-        if w_next is not None and (out is None or tuple(out.shape) != (n_out, width)):
+        if (w_next is not None or out is not None) and (out is None or tuple(out.shape) != (n_out, width)):
             raise KernelArgumentError("post_norm_add: the next norm needs an output of one row per taken row")
-        if w_next is None and rows is not None:
-            raise KernelArgumentError("post_norm_add: a row selection without a next norm has no result")
+        if out is None and rows is not None:
+            raise KernelArgumentError("post_norm_add: a row selection without an output has no result")
         _check(library().imparo_post_norm_add_moe(
             _dev(x, "stream", torch.float32), _dev(delta.y, "experts' results", torch.float32),
             _dev(delta.h, "feed-forward input", None, (n_x, width)), _code(delta.h, "feed-forward input"),
@@ -883,21 +904,21 @@ def post_norm_add(x: torch.Tensor, delta, w_post: torch.Tensor, eps_post: float,
             _dev(delta.slot_of_entry, "slot_of_entry", torch.int32, (n_x * top,)), top, int(delta.n_experts), n_x,
             _dev(rows, "rows", torch.int32), _dev(w_post, "post norm weight", torch.float32, (width,)), float(eps_post),
             _dev(w_next, "next norm weight", torch.float32, (width,)), float(eps_next),
-            _dev(out, "normed") if w_next is not None else None, _code(out, "normed") if w_next is not None else 0,
+            _dev(out, "normed"), _code(out, "normed") if out is not None else 0,
             n_out, width, _stream()), "post_norm_add")
         return out
     n_delta = delta.shape[0] if delta.dim() == 3 else 1
     _dev(delta, "sublayer result", torch.float32, ((n_delta, n_x, width) if delta.dim() == 3 else (n_x, width)))
-    if w_next is not None:
+    if w_next is not None or out is not None:
         if out is None or tuple(out.shape) != (n_out, width):
             raise KernelArgumentError("post_norm_add: the next norm needs an output of one row per taken row")
     elif rows is not None:
-        raise KernelArgumentError("post_norm_add: a row selection without a next norm has no result")
+        raise KernelArgumentError("post_norm_add: a row selection without an output has no result")
     _check(library().imparo_post_norm_add(
         _dev(x, "stream", torch.float32), delta.data_ptr(), n_delta, n_x, _dev(rows, "rows", torch.int32),
         _dev(w_post, "post norm weight", torch.float32, (width,)), float(eps_post),
         _dev(w_next, "next norm weight", torch.float32, (width,)), float(eps_next),
-        _dev(out, "normed") if w_next is not None else None, _code(out, "normed") if w_next is not None else 0,
+        _dev(out, "normed"), _code(out, "normed") if out is not None else 0,
         n_out, width, _stream()), "post_norm_add")
     return out
 
@@ -1110,3 +1131,146 @@ def add_rows(x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
     _check(library().imparo_add_rows(_dev(x, "x", torch.float32), _dev(y, "y", torch.float32, tuple(x.shape)),
                                      x.numel(), _stream()), "add_rows")
     return x
+
+
+# ---------------------------------------------------------------- recurrences with one decay a head and token
+DECAY_SCAN_MAX_DIM = 512          # state rows a head
+DECAY_SCAN_CHUNK = 64             # tokens a chunk when a long segment's chunks run side by side
+
+
+def decay_scan_chunks(max_seg_len: int, delta: bool = False):
+    """(chunk_tokens, max_chunks) for `decay_scan`: (0, 1) for one launch, which short segments and the delta
+    rule take; else chunks of DECAY_SCAN_CHUNK tokens, as many as the longest segment makes."""
+    if delta or max_seg_len < 4 * DECAY_SCAN_CHUNK:
+        return 0, 1
+    return DECAY_SCAN_CHUNK, -(-int(max_seg_len) // DECAY_SCAN_CHUNK)
+
+
+def decay_scan(q: torch.Tensor, q_off: int, q_div: int, k: torch.Tensor, k_off: int, k_div: int, v: torch.Tensor,
+               v_off: int, state: torch.Tensor, seg_start: torch.Tensor, seg_len: torch.Tensor, slot: torch.Tensor,
+               out: torch.Tensor, heads: int, dim: int, vdim: int, decay_const: Optional[torch.Tensor] = None,
+               step: Optional[torch.Tensor] = None, step_off: int = 0, step_bias: Optional[torch.Tensor] = None,
+               rate: Optional[torch.Tensor] = None, v_times_step: bool = False, beta: Optional[torch.Tensor] = None,
+               beta_off: int = 0, skip: Optional[torch.Tensor] = None, chunk_tokens: int = 0, max_chunks: int = 1,
+               chunk_state: Optional[torch.Tensor] = None, chunk_decay: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Per request, head and token in order: S <- a S + k v^T, out = S^T q; with `beta` the gated delta rule
+    S <- a S, u = sigmoid(beta) (v - S^T k), S <- S + k u^T, out = S^T q. q, k, v, step, beta are float32 row
+    tensors [tokens, ld] read from a column offset on (they may be one tensor); head h reads q head h // q_div
+    and k head h // k_div. a = decay_const[h] or exp(-rate[h] softplus(step[t, h] + step_bias[h])); with
+    `v_times_step` v is multiplied by that softplus; with `skip`, out += skip[h] v. state [slots, heads, dim,
+    vdim] float32 is carried on; out [tokens, heads * vdim] float32."""
+    n = out.shape[0]
+    n_rows = seg_start.shape[0]
+    if dim > DECAY_SCAN_MAX_DIM:
+        raise KernelArgumentError(f"decay_scan: up to {DECAY_SCAN_MAX_DIM} state rows a head, got {dim}")
+    for t, what in ((q, "q"), (k, "k"), (v, "v"), (step, "step"), (beta, "beta")):
+        if t is not None and (t.dim() != 2 or t.shape[0] != n):
+            raise KernelArgumentError(f"decay_scan: {what} is not a row tensor of {n} tokens")
+    if (decay_const is None) == (step is None):
+        raise KernelArgumentError("decay_scan: the decay is a constant a head or comes from projected steps")
+    if chunk_tokens:
+        if beta is not None:
+            raise KernelArgumentError("decay_scan: the delta rule is walked in one launch")
+        need_s, need_d = n_rows * max_chunks * heads * dim * vdim, n_rows * max_chunks * heads
+        if chunk_state is None or chunk_decay is None or chunk_state.numel() < need_s or chunk_decay.numel() < need_d:
+            raise KernelArgumentError("decay_scan: the scratch for the chunks' states is too small")
+    _check(library().imparo_decay_scan(
+        _dev(q, "scan q", torch.float32), q.shape[1], int(q_off), int(q_div),
+        _dev(k, "scan k", torch.float32), k.shape[1], int(k_off), int(k_div),
+        _dev(v, "scan v", torch.float32), v.shape[1], int(v_off),
+        _dev(decay_const, "decays", torch.float32, (heads,)),
+        _dev(step, "steps", torch.float32), 0 if step is None else step.shape[1], int(step_off),
+        _dev(step_bias, "step bias", torch.float32, (heads,)) if step is not None else 0,
+        _dev(rate, "decay rates", torch.float32, (heads,)) if step is not None else 0, int(bool(v_times_step)),
+        _dev(beta, "beta", torch.float32), 0 if beta is None else beta.shape[1], int(beta_off),
+        _dev(skip, "skip weights", torch.float32, (heads,)),
+        _dev(state, "scan state", torch.float32, (state.shape[0], heads, dim, vdim)),
+        _dev(seg_start, "seg_start", torch.int32, (n_rows,)), _dev(seg_len, "seg_len", torch.int32, (n_rows,)),
+        _dev(slot, "slot", torch.int32, (n_rows,)), _dev(out, "scan out", torch.float32, (n, heads * vdim)),
+        n_rows, heads, dim, vdim, int(chunk_tokens), int(max_chunks),
+        _dev(chunk_state, "chunk states", torch.float32) if chunk_tokens else 0,
+        _dev(chunk_decay, "chunk decays", torch.float32) if chunk_tokens else 0, _stream()), "decay_scan")
+    return out
+
+
+def head_prepare(rows: torch.Tensor, off: int, heads: int, dim: int, unit: bool = False, unit_eps: float = 0.0,
+                 inv_freq: Optional[torch.Tensor] = None, interleaved: bool = False,
+                 positions: Optional[torch.Tensor] = None, n_first: int = 0, scale_first: float = 1.0,
+                 scale_rest: float = 1.0) -> torch.Tensor:
+    """In place on float32 rows [tokens, ld]: each of the `heads` heads of `dim` columns from `off` on is made a
+    unit vector (x / sqrt(sum x^2 + unit_eps)) if `unit`, its first 2 len(inv_freq) dimensions are rotated by the
+    token's position (pairs (i, i + half), or neighbours if `interleaved`), and it is multiplied by scale_first
+    (heads below n_first) or scale_rest."""
+    n, ld = rows.shape
+    n_freq = 0 if inv_freq is None else inv_freq.shape[0]
+    if off < 0 or off + heads * dim > ld or 2 * n_freq > dim:
+        raise KernelArgumentError(f"head_prepare: {heads} heads of {dim} from column {off} in rows of {ld}, {n_freq} rotated pairs")
+    _check(library().imparo_head_prepare(
+        _dev(rows, "rows", torch.float32), ld, int(off), n, heads, dim, int(bool(unit)), float(unit_eps),
+        _dev(inv_freq, "inverse frequencies", torch.float32), n_freq, int(bool(interleaved)),
+        _dev(positions, "positions", torch.int32, (n,)) if n_freq else 0, int(n_first), float(scale_first),
+        float(scale_rest), _stream()), "head_prepare")
+    return rows
+
+
+def gated_group_norm(x: torch.Tensor, gate: Optional[torch.Tensor], gate_off: int, weight: Optional[torch.Tensor],
+                     groups: int, eps: float, out: torch.Tensor, gate_first: bool) -> torch.Tensor:
+    """A row of x (float32 [tokens, width]) in `groups` equal parts, g = silu(gate[t, gate_off + c]):
+    gate_first: (x g) / rms_part(x g) * weight; otherwise x / rms_part(x) * weight * g. weight [width] or None."""
+    n, width = x.shape
+    if gate is not None and (gate.dim() != 2 or gate.shape[0] != n or gate_off + width > gate.shape[1]):
+        raise KernelArgumentError("gated_group_norm: the gate's rows do not hold the row's width from its offset on")
+    _check(library().imparo_gated_group_norm(
+        _dev(x, "heads' results", torch.float32), _dev(gate, "gate", torch.float32), 0 if gate is None else gate.shape[1],
+        int(gate_off), _dev(weight, "norm weight", torch.float32, (width,)), _dev(out, "normed", None, (n, width)),
+        _code(out, "normed"), n, width, int(groups), float(eps), int(bool(gate_first)), _stream()), "gated_group_norm")
+    return out
+
+
+def clamped_glu(gu: torch.Tensor, out: torch.Tensor, hidden: int, limit: float, alpha: float) -> torch.Tensor:
+    """out[t, j] = g sigmoid(alpha g) (u + 1) with g = min(gu[t, j], limit), u = clamp(gu[t, hidden + j], -limit,
+    limit); out may be wider than `hidden` (its further columns are zero)."""
+    n = gu.shape[0]
+    if gu.shape[1] != 2 * hidden or out.shape[0] != n or out.shape[1] < hidden:
+        raise KernelArgumentError(f"clamped_glu: gu is {tuple(gu.shape)}, out {tuple(out.shape)}, hidden {hidden}")
+    _check(library().imparo_clamped_glu(_dev(gu, "gate and up", torch.float32), _dev(out, "hidden"), _code(out, "hidden"),
+                                        n, int(hidden), out.shape[1], float(limit), float(alpha), _stream()), "clamped_glu")
+    return out
+
+
+def normed_sum(a: torch.Tensor, wa: torch.Tensor, b: torch.Tensor, wb: torch.Tensor, eps: float, factor: float,
+               out: torch.Tensor) -> torch.Tensor:
+    """out = factor (rms_norm(a) wa + rms_norm(b) wb); a and b float32 [tokens, width] or [slices, tokens, width]
+    (slices are added in order first)."""
+    n, width = out.shape
+    sa = a.shape[0] if a.dim() == 3 else 1
+    sb = b.shape[0] if b.dim() == 3 else 1
+    _dev(a, "first result", torch.float32, (sa, n, width) if a.dim() == 3 else (n, width))
+    _dev(b, "second result", torch.float32, (sb, n, width) if b.dim() == 3 else (n, width))
+    _check(library().imparo_normed_sum(a.data_ptr(), sa, _dev(wa, "first weight", torch.float32, (width,)), b.data_ptr(), sb,
+                                       _dev(wb, "second weight", torch.float32, (width,)),
+                                       _dev(out, "sum", torch.float32), n, width, float(eps), float(factor), _stream()),
+           "normed_sum")
+    return out
+
+
+def gated_row_add(out: torch.Tensor, y: torch.Tensor, z: torch.Tensor, z_col: int) -> torch.Tensor:
+    """out[t] += sigmoid(z[t, z_col]) * y[t]; y float32 [tokens, width] or [slices, tokens, width]."""
+    n, width = out.shape
+    sy = y.shape[0] if y.dim() == 3 else 1
+    _dev(y, "rows to add", torch.float32, (sy, n, width) if y.dim() == 3 else (n, width))
+    if z.dim() != 2 or z.shape[0] != n or not 0 <= z_col < z.shape[1]:
+        raise KernelArgumentError("gated_row_add: one gate a token is read from a column of z")
+    _check(library().imparo_gated_row_add(_dev(out, "sum", torch.float32), y.data_ptr(), sy, _dev(z, "gates", torch.float32),
+                                          z.shape[1], int(z_col), n, width, _stream()), "gated_row_add")
+    return out
+
+
+def cast_rows(x: torch.Tensor, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[i] = x[rows[i]] (rows None: x[i]) in out's dtype; x float32 [n, width]."""
+    n_out, width = out.shape
+    if x.shape[1] != width or (rows is None and x.shape[0] != n_out) or (rows is not None and rows.shape[0] != n_out):
+        raise KernelArgumentError(f"cast_rows: x is {tuple(x.shape)}, out {tuple(out.shape)}")
+    _check(library().imparo_cast_rows(_dev(x, "rows", torch.float32), _dev(rows, "row choice", torch.int32),
+                                      _dev(out, "cast rows"), _code(out, "cast rows"), n_out, width, _stream()), "cast_rows")
+    return out

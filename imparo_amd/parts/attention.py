@@ -13,6 +13,14 @@ layer's cache looks further back than this layer itself; None: everything),
 `shared_kv` (the layer has no key and value projections: it is run with
 another layer's cache, `LayerCall.cache_of`, and brings queries only),
 `weight_suffix` and `names` (how the checkpoint calls the tensors),
+`chunk` (instead of a window: a query at position i sees j <= i only in its
+own chunk, floor(i / chunk) = floor(j / chunk), chunks counted from position 0
+whatever way a prompt was cut), `bias` (q, k, v and the output projection carry
+biases, the tensor's name with `bias_suffix`, added in the projection),
+`conv_taps` (a causal convolution per channel on q, k and v right behind the
+projection, before head norm and rotation: y_t = sum_j w[:, j] u_(t - taps + 1 + j),
+no bias, zeros before the start, tensors `<name>.conv`; the last taps - 1
+projected rows of a request are state beside its pages),
 `exact_weights` (the softmax weights keep float32's precision through the
 product with the values: the matrix-core kernels then send what rounding a
 weight to bfloat16 took off through a second product; the wave kernel, which
@@ -23,7 +31,7 @@ from typing import Dict, Optional
 
 import torch
 
-from ..cache.pages import PagedSpec, kv_spec
+from ..cache.pages import FixedArray, PagedSpec, kv_spec, with_fixed_arrays
 from ..config.plan import PartSpec
 from ..kernels import ops
 from ..weights.loader import TensorDecl
@@ -60,6 +68,16 @@ class Attention:
             out[n["q_norm"] + sfx] = (TensorDecl((D,), "vector"), "norm")
             if not shared:
                 out[n["k_norm"] + sfx] = (TensorDecl((D,), "vector"), "norm")
+        sides = ("q",) if shared else ("q", "k", "v")
+        rows = dict(q=H * D, k=Hk * D, v=Hk * Dv)
+        if spec.get("bias"):
+            bsfx = spec.get("bias_suffix", ".bias")
+            for x in sides:
+                out[n[x] + bsfx] = (TensorDecl((rows[x],), "vector"), "bias")
+            out[n["o"] + bsfx] = (TensorDecl((E,), "vector"), "bias")
+        if spec.get("conv_taps"):
+            for x in sides:
+                out[n[x] + spec.get("conv_suffix", ".conv")] = (TensorDecl((rows[x], spec["conv_taps"]), "vector"), "conv")
         return out
 
     def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], device: torch.device,
@@ -78,11 +96,30 @@ class Attention:
         self.scale = float(spec["scale"])
         self.window: Optional[int] = spec.get("window")
         self.keep_window: Optional[int] = spec.params["keep_window"] if "keep_window" in spec.params else self.window
-        ws = [tensors[n[x] + sfx] for x in (("q",) if self.shared_kv else ("q", "k", "v"))]
+        self.chunk: Optional[int] = spec.get("chunk")
+        if self.chunk is not None:
+            if self.window is not None or self.keep_window is not None or self.chunk < 1:
+                raise ValueError("a layer sees a window or its own chunk (of at least one position), not both")
+            self.window = -int(self.chunk)        # as the kernels take it: a negative window is a chunk of that size
+        sides = ("q",) if self.shared_kv else ("q", "k", "v")
+        ws = [tensors[n[x] + sfx] for x in sides]
         if len({w.dtype for w in ws}) > 1:
             ws = [w.to(torch.float32) for w in ws]
+        bias = out_bias = None
+        if spec.get("bias"):
+            bsfx = spec.get("bias_suffix", ".bias")
+            bias = place_vector(torch.cat([tensors[n[x] + bsfx].to(torch.float32) for x in sides]), device)
+            out_bias = place_vector(tensors[n["o"] + bsfx], device)
         # one projection for q | k | v: the same dot products, one launch
-        self.qkv = Linear(place_projection(torch.cat(ws, dim=0), engine_dtype, device))
+        self.qkv = Linear(place_projection(torch.cat(ws, dim=0), engine_dtype, device), bias)
+        self.conv_taps = int(spec.get("conv_taps") or 0)
+        self.conv_weight = None
+        if self.conv_taps:
+            if self.conv_taps > 64:
+                raise ValueError(f"the conv kernels take at most 64 taps, got {self.conv_taps}")
+            csfx = spec.get("conv_suffix", ".conv")
+            self.conv_weight = place_vector(torch.cat([tensors[n[x] + csfx].to(torch.float32).reshape(-1, self.conv_taps)
+                                                       for x in sides], dim=0), device)
         out = tensors[n["o"] + sfx]
         # The attention kernels write their result in the cache's dtype and the bfloat16 products walk K in steps
         # of 8: where heads x value size is no multiple of 8 the output projection gets columns of zero weight and
@@ -90,7 +127,7 @@ class Attention:
         self.out_fill = (-self.heads * self.value_dim) % 8 if engine_dtype != torch.float32 and out.dtype != torch.float32 else 0
         if self.out_fill:
             out = torch.cat([out, out.new_zeros(out.shape[0], self.out_fill)], dim=1)
-        self.out = Linear(place_matrix(out, engine_dtype, device))
+        self.out = Linear(place_matrix(out, engine_dtype, device), out_bias)
         norm = spec.get("qk_norm")
         if norm is not None:
             # the kernels that norm a head know one norm: RMS with a weight per dimension, no offset
@@ -118,7 +155,10 @@ class Attention:
         16, head sizes up to 128), V is kept transposed inside a page."""
         self.v_transposed = (self.value_dim == self.head_dim
                              and ops.mfma_attention_supported(self.engine_dtype, page_size, self.head_dim))
-        return kv_spec(self.kv_heads, self.head_dim, self.keep_window, self.v_transposed, self.value_dim)
+        spec = kv_spec(self.kv_heads, self.head_dim, self.keep_window, self.v_transposed, self.value_dim, self.chunk)
+        if self.conv_taps > 1:
+            spec = with_fixed_arrays(spec, (FixedArray("conv", (self.conv_taps - 1, self.qkv.out_features), "float32", 0.0),))
+        return spec
 
     def _portion_tiles(self, ctx: StepContext) -> int:
         """Tiles of queries that the portions of this batch make, as the prompt kernel counts them."""
@@ -142,6 +182,13 @@ class Attention:
         if self.shared_kv and owns_cache:
             raise ValueError("a layer without key and value projections must be run with another layer's cache")
         qkv = self.qkv(ctx, h, torch.float32, "qkv", alias="mixer_in")
+        if self.conv_taps:
+            if not owns_cache:
+                raise ValueError("a conv's history cannot be read from another layer")
+            mixed = ctx.workspace.get("qkv_conv", tuple(qkv.shape), torch.float32)
+            history = ctx.fixed_arrays(site)["conv"] if self.conv_taps > 1 else None
+            qkv = ops.causal_conv(qkv, qkv.shape[1], self.conv_weight, None, history, ctx.row_of_token, ctx.seg_start,
+                                  ctx.seg_len, ctx.slot, mixed, silu=False, single_tokens=ctx.max_seg_len == 1)
         k_cache, v_cache, table = ctx.kv(site)
         vt = self.v_transposed
         inv_freq = self.position.inv_freq
@@ -199,7 +246,7 @@ class Attention:
     def can_emit(self) -> bool:
         # the step program's attention has one head size, keys and values of its own, and the matrix-core kernels
         return (self.value_dim == self.head_dim and not self.shared_kv and not self.exact_weights
-                and not self.out_fill)
+                and not self.out_fill and not self.conv_taps and self.chunk is None)
 
     def emit(self, program, site: int, owns_cache: bool) -> None:
         """Appends `forward` to a native step program."""

@@ -47,6 +47,8 @@ class SwiGlu:
         n = self._names(spec)
         sfx = spec.get("weight_suffix", ".weight")          # what a checkpoint appends to a matrix's name
         self.width, self.hidden = spec["width"], spec["hidden"]
+        # a second feed-forward inside another part keeps its scratch under names of its own
+        self.tag = spec.get("scratch_tag") or ""
         gate, up = tensors[n["gate"] + sfx], tensors[n["up"] + sfx]
         if gate.dtype != up.dtype:
             gate, up = gate.to(torch.float32), up.to(torch.float32)
@@ -71,10 +73,13 @@ class SwiGlu:
 
     def forward(self, ctx: StepContext, n: torch.Tensor) -> torch.Tensor:
         # the gated hidden may lie where the mixer's input projection lay: that is dead by now
-        g = self.gate_up(ctx, n, self.down.in_dtype, "gated", swiglu=True, alias="mixer_in")
+        g = self.gate_up(ctx, n, self.down.in_dtype, self.tag + "gated", swiglu=True, alias="mixer_in")
         # the result is a delta for the residual stream, whose next norm adds slices: it may come sliced
-        return self.down(ctx, g, torch.float32, "ffn_out", sliced_ok=True, into=ctx.stream)
+        return self.down(ctx, g, torch.float32, self.tag + "ffn_out", sliced_ok=True, into=ctx.stream)
 
+
+    def can_emit(self) -> bool:
+        return not self.tag
 
     def emit(self, program) -> None:
         """Appends `forward` to a native step program."""
@@ -129,5 +134,50 @@ class PolyNormFfn:
         return self.down(ctx, g, torch.float32, "ffn_out", sliced_ok=True, into=ctx.stream)
 
 
+class ClampedGlu:
+    """A gated unit with bounds: g = min(Wgate n, limit), u = clamp(Wup n, -limit, limit),
+    f = Wdown (g sigmoid(alpha g) (u + 1)). Parameters: width, hidden, limit, alpha (1.702 unless
+    given), names, weight_suffix."""
+    role = "feed_forward"
+    graph_safe = True     # launches kernels only: a step made of such parts can be captured
+    _names = staticmethod(SwiGlu._names)
+
+    @classmethod
+    def declare(cls, spec: PartSpec) -> Declared:
+        return SwiGlu.declare.__func__(cls, spec)
+
+    def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], device: torch.device,
+                 engine_dtype: torch.dtype):
+        n = self._names(spec)
+        sfx = spec.get("weight_suffix", ".weight")
+        self.width, self.hidden = spec["width"], spec["hidden"]
+        self.limit = float(spec["limit"])
+        self.alpha = float(spec.get("alpha", 1.702))
+        if not self.limit > 0:
+            raise ValueError(f"the bound of a clamped unit is positive, got {self.limit}")
+        gate, up, down = tensors[n["gate"] + sfx], tensors[n["up"] + sfx], tensors[n["down"] + sfx]
+        if gate.dtype != up.dtype:
+            gate, up = gate.to(torch.float32), up.to(torch.float32)
+        # one projection for gate | up (gate rows first); the activation reads both halves of its float32 rows.
+        # The bfloat16 kernels walk K in steps of 8: a hidden width that is none gets columns of zero weight on the
+        # way back, and the activation fills the hidden rows up with zeros.
+        self.fill = (-self.hidden) % 8 if engine_dtype != torch.float32 and down.dtype != torch.float32 else 0
+        if self.fill:
+            down = torch.cat([down, down.new_zeros(self.width, self.fill)], dim=1)
+        self.gate_up = Linear(place_projection(torch.cat([gate, up], dim=0), engine_dtype, device))
+        self.down = Linear(place_matrix(down, engine_dtype, device))
+
+    @property
+    def in_dtype(self) -> torch.dtype:
+        return self.gate_up.in_dtype
+
+    def forward(self, ctx: StepContext, n: torch.Tensor) -> torch.Tensor:
+        gu = self.gate_up(ctx, n, torch.float32, "gate_up", alias="mixer_in")
+        g = ctx.workspace.get("gated", (n.shape[0], self.hidden + self.fill), self.down.in_dtype, alias="mixer_mid")
+        ops.clamped_glu(gu, g, self.hidden, self.limit, self.alpha)
+        return self.down(ctx, g, torch.float32, "ffn_out", sliced_ok=True, into=ctx.stream)
+
+
 register_part("feed_forward", "swiglu", SwiGlu)
+register_part("feed_forward", "clamped_glu", ClampedGlu)
 register_part("feed_forward", "poly_norm", PolyNormFfn)

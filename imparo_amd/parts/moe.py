@@ -15,7 +15,14 @@ Parameters: width, hidden (an expert's), experts, identity, top, activation
 scoring ("softmax" over all router outputs, or "sigmoid" of each output by
 itself), weigh ("output": a chosen expert's result is multiplied by its
 weight; "input": the expert reads its input times its weight and the results
-are added as they are), and the tensors' names: `router`, `correction` (None:
+are added as they are), `group_count` and `group_keep` (the router outputs form
+group_count equal groups of neighbours; a group's score is the sum of its two
+largest score + correction, and only outputs of the group_keep best groups can
+be chosen: the others' choice scores count as minus infinity), `normalize` (the
+chosen scores are divided by their sum + 1e-20), `route_scale` (a factor on the
+weights), `shared` (the PartSpec of a feed-forward that every token uses; its
+result is added, multiplied by sigmoid(Wsg n), one number a token, with Wsg the
+tensor `shared_gate`), and the tensors' names: `router`, `correction` (None:
 no correction), `expert_up` / `expert_down` as patterns with `{e}` for the
 expert's number.
 
@@ -26,7 +33,7 @@ nothing comes back to the host and a step of this part can be captured.
 """
 from __future__ import annotations
 
-from typing import Dict
+from typing import Dict, Optional
 
 import torch
 
@@ -35,7 +42,7 @@ from ..kernels import ops
 from ..weights.loader import TensorDecl
 from .base import Declared, RowsToCombine, StepContext
 from .linear import Linear, place_matrix, place_projection, place_vector
-from .registry import register_part
+from .registry import part_class, register_part
 
 
 class RoutedExperts:
@@ -45,7 +52,7 @@ class RoutedExperts:
     @staticmethod
     def _names(spec: PartSpec) -> Dict[str, str]:
         names = dict(router="router", correction="correction", expert_up="e{e}.up", expert_down="e{e}.down",
-                     expert_gate="e{e}.gate")
+                     expert_gate="e{e}.gate", shared_gate="shared.sg")
         names.update(spec.get("names") or {})
         return {k: (None if v is None else f"{spec.prefix}.{v}") for k, v in names.items()}
 
@@ -61,6 +68,9 @@ class RoutedExperts:
                 out[n["expert_gate"].format(e=e)] = (TensorDecl((F, E)), "matrix")
             out[n["expert_up"].format(e=e)] = (TensorDecl((F, E)), "matrix")
             out[n["expert_down"].format(e=e)] = (TensorDecl((E, F)), "matrix")
+        if spec.get("shared") is not None:
+            out.update(part_class("feed_forward", spec["shared"].kind).declare(spec["shared"]))
+            out[n["shared_gate"]] = (TensorDecl((1, E)), "matrix")
         return out
 
     def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], device: torch.device,
@@ -85,7 +95,27 @@ class RoutedExperts:
             raise ValueError(f"{self.top} of {self.experts + self.identity} experts cannot be chosen")
         # bfloat16 x bfloat16 products are exact in float32 and the sums are float32: the router runs in 32 bits
         # on the matrix cores too; its input is the norm's output in the engine's dtype
-        self.router = Linear(place_projection(tensors[n["router"]], engine_dtype, device))
+        self.n_router = self.experts + self.identity
+        self.group_count, self.group_keep = int(spec.get("group_count") or 1), int(spec.get("group_keep") or 1)
+        if self.group_count > 1 and (self.n_router % self.group_count or not 1 <= self.group_keep <= self.group_count
+                                     or self.group_keep * (self.n_router // self.group_count) < self.top):
+            raise ValueError(f"{self.n_router} router outputs in {self.group_count} groups of which {self.group_keep} "
+                             f"stay cannot give {self.top} choices")
+        self.normalize, self.route_scale = bool(spec.get("normalize")), float(spec.get("route_scale", 1.0))
+        router = tensors[n["router"]]
+        self.shared = None
+        if spec.get("shared") is not None:
+            if self.top > 0 and spec["shared"].get("scratch_tag") is None:
+                raise ValueError("a feed-forward inside this one keeps its scratch under a tag of its own (scratch_tag)")
+            self.shared = part_class("feed_forward", spec["shared"].kind)(spec["shared"], tensors, device, engine_dtype)
+            # the shared expert's gate is one more row of the router's matrix: the same dot products, one launch
+            gate = tensors[n["shared_gate"]].reshape(1, self.width)
+            if gate.dtype != router.dtype:
+                router, gate = router.to(torch.float32), gate.to(torch.float32)
+            router = torch.cat([router, gate], dim=0)
+        self.router = Linear(place_projection(router, engine_dtype, device))
+        if self.shared is not None and self.shared.in_dtype != self.router.in_dtype:
+            raise ValueError("the shared expert and the router read their input in one dtype")
         self.correction = None if n["correction"] is None else place_vector(tensors[n["correction"]], device)
         ups = [tensors[n["expert_up"].format(e=e)] for e in range(self.experts)]
         downs = [tensors[n["expert_down"].format(e=e)] for e in range(self.experts)]
@@ -115,12 +145,27 @@ class RoutedExperts:
     def in_dtype(self) -> torch.dtype:
         return self.router.in_dtype
 
-    def forward_rows(self, ctx: StepContext, n: torch.Tensor) -> RowsToCombine:
+    @property
+    def forward_rows(self):
         """Everything but the weighted sum over a token's experts: for a block whose next launch (a norm on
-        this part's result) makes that sum itself."""
+        this part's result) makes that sum itself. None where the result is more than that sum."""
+        return None if self.shared is not None else self._rows
+
+    def _rows(self, ctx: StepContext, n: torch.Tensor, shared_out: Optional[list] = None) -> RowsToCombine:
         T, top, X = n.shape[0], self.top, self.experts
         ws = ctx.workspace
+        rules = dict(scoring=self.scoring, n_router=self.n_router, groups=self.group_count, keep=self.group_keep,
+                     normalize=self.normalize, scale=self.route_scale)
+        if self.shared is not None:
+            # first, while the scratch it shares with the experts' products is free
+            stream, ctx.stream = ctx.stream, None          # (its result is weighed before it is added anywhere)
+            try:
+                shared_out.append(self.shared.forward(ctx, n))
+            finally:
+                ctx.stream = stream
         z = self.router(ctx, n, torch.float32, "router_logits")
+        if shared_out is not None:
+            shared_out.append(z)
         choice = ws.get("moe_choice", (T, top), torch.int32)
         weight = ws.get("moe_weight", (T, top), torch.float32)
         entries = T * top
@@ -132,9 +177,9 @@ class RoutedExperts:
             entry_of_slot = ws.get("moe_entry_of_slot", (entries,), torch.int32)
             if T <= ops.moe_route_plan_tokens():      # a decode step: choice and plan in one launch
                 ops.moe_route_plan(z, self.correction, choice, weight, top, X, rows, slot_of_entry, entry_of_slot, tiles,
-                                   scoring=self.scoring)
+                                   **rules)
             else:
-                ops.moe_route(z, self.correction, choice, weight, top, scoring=self.scoring)
+                ops.moe_route(z, self.correction, choice, weight, top, **rules)
                 ops.moe_plan(choice, X, rows, slot_of_entry, entry_of_slot, tiles)
             if self.gated:
                 both = ws.get("moe_gate_up", (entries, self.up.shape[1]), torch.float32, alias="mixer_in")
@@ -146,13 +191,18 @@ class RoutedExperts:
                 ops.moe_gemm(n, self.up, hidden, tiles, rows, entry_of_slot, gather_div=top, epilogue=self.activation)
             ops.moe_gemm(hidden, self.down, y, tiles, rows)
         else:
-            ops.moe_route(z, self.correction, choice, weight, top, scoring=self.scoring)
+            ops.moe_route(z, self.correction, choice, weight, top, **rules)
         return RowsToCombine(y, n, choice, None if self.weigh == "input" else weight, slot_of_entry, X)
 
     def forward(self, ctx: StepContext, n: torch.Tensor) -> torch.Tensor:
-        r = self.forward_rows(ctx, n)
+        extra: list = []
+        r = self._rows(ctx, n, extra if self.shared is not None else None)
         out = ctx.workspace.get("ffn_out", (n.shape[0], self.width), torch.float32)
-        return ops.moe_combine(r.y, r.h, r.choice, r.weight, r.slot_of_entry, r.n_experts, out)
+        ops.moe_combine(r.y, r.h, r.choice, r.weight, r.slot_of_entry, r.n_experts, out)
+        if self.shared is not None:
+            y, z = extra
+            ops.gated_row_add(out, y, z, self.n_router)
+        return out
 
 
 register_part("feed_forward", "routed_experts", RoutedExperts)

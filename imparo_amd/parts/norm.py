@@ -130,4 +130,54 @@ class RmsNorm:
         return out
 
 
+class NoNorm:
+    """No norm where a block has a place for one: the sublayer reads the stream itself. What is
+    pending on the stream is added first, through the norm it carries if it carries one, in the
+    same launch that hands the rows on in the dtype the reader asks for."""
+    role = "norm"
+    graph_safe = True     # launches kernels only: a step made of such parts can be captured
+
+    @classmethod
+    def declare(cls, spec: PartSpec) -> Declared:
+        return {}
+
+    def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], device: torch.device,
+                 engine_dtype: torch.dtype):
+        self.width = spec["width"]
+
+    @staticmethod
+    def _add_plain(res: Residual, pending) -> None:
+        """A delta that carries no norm: its slices are added to the stream in order."""
+        if not isinstance(pending, torch.Tensor):
+            raise ValueError("rows that a routed feed-forward left to be combined go through a norm behind it")
+        for part in (pending if pending.dim() == res.x.dim() + 1 else [pending]):
+            ops.add_rows(res.x, part)
+
+    def forward(self, ctx: StepContext, res: Residual, out_dtype: torch.dtype, name: str = "normed") -> torch.Tensor:
+        pending, res.pending = res.pending, None
+        post, res.post = res.post, None
+        if pending is not None and post is None:
+            self._add_plain(res, pending)
+            pending = None
+        if pending is None and out_dtype == torch.float32:
+            return res.x          # readers do not write into what they read
+        out = ctx.workspace.get(name, tuple(res.x.shape), out_dtype)
+        if pending is None:
+            return ops.cast_rows(res.x, out)
+        ops.post_norm_add(res.x, pending, post[0], post[1], None, 0.0, out)
+        return out
+
+    def forward_rows(self, ctx: StepContext, res: Residual, rows: torch.Tensor, out_dtype: torch.dtype,
+                     name: str = "normed_rows") -> torch.Tensor:
+        """The chosen rows as they would be after the pending add; the stream itself is left as it is."""
+        out = ctx.workspace.get(name, (rows.shape[0], self.width), out_dtype)
+        if res.pending is None:
+            return ops.cast_rows(res.x, out, rows)
+        if res.post is None:
+            raise ValueError("rows are chosen from a stream whose pending delta goes through a norm, or has none pending")
+        ops.post_norm_add(res.x, res.pending, res.post[0], res.post[1], None, 0.0, out, rows=rows)
+        return out
+
+
 register_part("norm", "rms_norm", RmsNorm)
+register_part("norm", "none", NoNorm)
