@@ -441,6 +441,29 @@ def kosalorn_shape(width, heads, expert_ff, dense_ff, experts=8, top=4, layers=1
                 layers=[dict(run[i % 4]) for i in range(layers)])
 
 
+def mepapel_shape(width, heads, expert_ff, dense_ff, experts=8, top=4, layers=16, chunk=8192):
+    """A Mepapel model of the width, heads and depth of the Kosalorn shape above, in a run of four layers: the gated
+    delta rule (heads of 128 by 128, two heads a query/key head) over a dense feed-forward, attention in chunks (heads
+    of 64, rotated whole, a short conv on q, k and v; chunks as long as the benchmark's longest prompt, so every cached
+    key is read) beside retention (heads of 128 by 128) over a mixture of experts, a state-space layer (inner 2 x
+    width in heads of 64, 128 state rows) over a dense feed-forward, and the delta rule over the experts. Gated
+    experts of three matrices each, `top` of `experts` a token out of three of four groups, and a shared expert."""
+    wide = width // 128
+    delta = dict(type="delta", mixer=dict(heads=wide, kv_heads=wide // 2, dim=128, vdim=128, conv=4))
+    pair = dict(type="parallel", mixer=dict(
+        left=dict(heads=heads, kv_heads=8, dim=64, vdim=64, scale=0.125, conv=4, mask=dict(size=chunk),
+                  rot=dict(dims=64, base=1000000.0)),
+        right=dict(heads=wide, dim=128, vdim=128, decay=[1.0 - 2.0 ** (-5 - 5 * i / max(wide - 1, 1)) for i in range(wide)],
+                   rot=dict(dims=64, base=10000.0))))
+    ssd = dict(type="mamba2", mixer=dict(heads=2 * width // 64, vdim=64, state=128, groups=1, norm_groups=1, conv=4))
+    moe = dict(kind="moe", expert=dict(ff=expert_ff), shared=dict(ff=expert_ff),
+               router=dict(experts=experts, top=top, scale=2.5, groups=dict(count=4, keep=3)))
+    dense = dict(kind="dense", ff=dense_ff, limit=7.0)
+    run = [dict(delta, mlp=dense), dict(pair, mlp=moe), dict(ssd, mlp=dense), dict(delta, mlp=moe)]
+    return dict(architecture="Mepapel", vocab=65536, width=width, norm=dict(eps=1e-5), residual_mult=0.5,
+                layers=[dict(run[i % 4]) for i in range(layers)])
+
+
 def compare_workload(workload, sizes, dtype, steps, warmup, beside="lfm2"):
     """Prefill and decode throughput of one design at some sizes, beside the closest model the engine has
     (`beside`: LFM2 unless said) at equal layer sizes, through the same loops. `sizes`: (name, that model's
@@ -510,6 +533,18 @@ def kosalorn_workload(dtype, steps, warmup, only=None, alone=False):
     return compare_workload("kosalorn", sizes, dtype, steps, warmup, beside="pupalorn")
 
 
+def mepapel_workload(dtype, steps, warmup, only=None, alone=False):
+    """The Mepapel design at two sizes beside Kosalorn, the engine's closest model (attention over a paged cache in
+    some layers, a recurrence with a matrix of state a head in others, a mixture of gated experts), at equal width,
+    heads and depth. `only`: one size; `alone`: without Kosalorn."""
+    sizes = [
+        ("1.2B", kosalorn_shape(2048, 32, 1408, 5632), mepapel_shape(2048, 32, 1408, 5632)),
+        ("350M", kosalorn_shape(1024, 16, 768, 3072), mepapel_shape(1024, 16, 768, 3072)),
+    ]
+    sizes = [(n, None if alone else a, b) for n, a, b in sizes if only in (None, n)]
+    return compare_workload("mepapel", sizes, dtype, steps, warmup, beside="kosalorn")
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -521,14 +556,15 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64 and the prefill")
     ap.add_argument("--prefill-only", action="store_true", help="run only the 2,048-token prefill (for profiling)")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "long", "tumadra", "pupalorn", "kosalorn"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "long", "tumadra", "pupalorn", "kosalorn", "mepapel"],
                     help="decode: the headline line (default). serving: continuous batching of 32 requests in 4 "
                          "waves (LFM2-700M shape). long: 64 requests of 32,768-token prompts, then 128 tokens "
                          "each (LFM2-350M shape). tumadra: prefill and decode of the Tumadra design at two sizes "
                          "beside LFM2 at equal size; pupalorn: the same for the Pupalorn design; kosalorn: the "
-                         "Kosalorn design beside Pupalorn. All but the first print a line of their own")
-    ap.add_argument("--size", default=None, choices=["1.2B", "350M"], help="--workload pupalorn or kosalorn: one size only")
-    ap.add_argument("--alone", action="store_true", help="--workload pupalorn or kosalorn: without the other model's runs beside it")
+                         "Kosalorn design beside Pupalorn; mepapel: the Mepapel design beside Kosalorn. All but the first print "
+                         "a line of their own")
+    ap.add_argument("--size", default=None, choices=["1.2B", "350M"], help="--workload pupalorn, kosalorn or mepapel: one size only")
+    ap.add_argument("--alone", action="store_true", help="--workload pupalorn, kosalorn or mepapel: without the other model's runs beside it")
     ap.add_argument("--requests", type=int, default=64, help="--workload long: concurrent requests")
     ap.add_argument("--prompt-len", type=int, default=32768, help="--workload long: tokens per prompt")
     ap.add_argument("--portion", type=int, default=2048, help="--workload long: tokens of a prompt per step")
@@ -547,6 +583,9 @@ def main() -> int:
         return 0
     if args.workload == "pupalorn":
         print(json.dumps(pupalorn_workload(args.dtype, args.steps, args.warmup, args.size, args.alone)), flush=True)
+        return 0
+    if args.workload == "mepapel":
+        print(json.dumps(mepapel_workload(args.dtype, args.steps, args.warmup, args.size, args.alone)), flush=True)
         return 0
     if args.workload == "kosalorn":
         print(json.dumps(kosalorn_workload(args.dtype, args.steps, args.warmup, args.size, args.alone)), flush=True)

@@ -178,9 +178,14 @@ int imparo_hgrn2_scan(const float* rows, int ld, int q_off, int f_off, int v_off
 // floats apart, heads from off on; head h reads q head h / q_div and k head h / k_div). a = decay_const[h], or
 // exp(-rate[h] softplus(step[t, h] + step_bias[h])); with v_times_step v is multiplied by that softplus; with
 // `skip`, out += skip[h] v (v as it came). state [slots, heads, dim, vdim] float32; out [tokens, heads * vdim]
-// float32. dim <= 512. chunk_tokens 0: one launch. Otherwise (a multiple of 8, not with beta) segments are walked
+// float32. dim <= 512. chunk_tokens 0: one launch. Otherwise (a multiple of 8; without beta) segments are walked
 // in chunks side by side, in three launches; max_chunks >= ceil(longest segment / chunk_tokens); chunk_state
 // [n_rows * max_chunks, heads, dim, vdim] and chunk_decay [n_rows * max_chunks, heads] float32 are scratch.
+// With beta, chunk_tokens is 0 or imparo_delta_chunk_tokens() (dim at most imparo_delta_chunk_max_dim()): the delta
+// rule in chunks, two launches; chunk_state then holds [n_rows * max_chunks, heads, 2, chunk, chunk] floats and
+// chunk_decay [n_rows * max_chunks, heads, chunk].
+int imparo_delta_chunk_tokens(void);
+int imparo_delta_chunk_max_dim(void);
 int imparo_decay_scan(const float* q, int q_ld, int q_off, int q_div, const float* k, int k_ld, int k_off, int k_div,
                       const float* v, int v_ld, int v_off, const float* decay_const, const float* step, int step_ld,
                       int step_off, const float* step_bias, const float* rate, int v_times_step, const float* beta,

@@ -186,6 +186,194 @@ __global__ void k_decay_carry(float* __restrict__ chunk_state, const float* __re
     }
 }
 
+// ---------------------------------------------------------------- the delta rule in chunks
+// Inside a chunk of DC tokens that starts from the state S0, with g_t the product of the decays from the
+// chunk's start up to token t:
+//   u_t = b_t (v_t - g_t S0^T k_t - sum_{j<t} (g_t / g_j) (k_t . k_j) u_j)        (I + L) U = diag(b) (V - P),
+//   o_t = g_t S0^T q_t + sum_{j<=t} (g_t / g_j) (q_t . k_j) u_j                     O = Qs + M U,
+//   S_end = g_last S0 + sum_j (g_last / g_j) k_j u_j^T.
+// A first launch makes, for every chunk of every segment and head side by side, T = (I + L)^-1 diag(b) (a lower
+// triangle, by forward substitution, a column a thread), M and the logarithms of g (sums of -rate * step, so
+// that every ratio is the exponential of a difference and at most one). A second launch walks a segment's
+// chunks in order with the state in LDS, a block a (segment, head, run of DVB value columns): four small
+// products a chunk on the vector units, every sum in an order the sizes alone decide. Tokens past a segment's
+// end count as k = q = 0, b = 0 and a decay of one: they change nothing.
+#define DC 32                 // tokens a chunk
+#define DVB 32                // value columns a block of the walk
+#define DMAXK 128             // state rows a head at most, in this form
+
+__global__ __launch_bounds__(256) void k_delta_chunk_prepare(const DecayScanArgs A) {
+    __shared__ float sk[DC][DMAXK + 1], sq[DC][DMAXK + 1], sL[DC][DC + 1], lg[DC], sb[DC];
+    const int r = blockIdx.x / A.max_chunks, chunk = blockIdx.x - r * A.max_chunks, h = blockIdx.y;
+    const int tid = threadIdx.x, dim = A.dim, heads = A.heads;
+    const int n_all = A.seg_len[r];
+    if (chunk * DC >= n_all) return;                     // (the whole block)
+    const int first = A.seg_start[r] + chunk * DC, n = min(DC, n_all - chunk * DC);
+    const int qh = h / A.q_div, kh = h / A.k_div;
+    for (int i = tid; i < DC * dim; i += 256) {
+        const int t = i / dim, k = i - t * dim;
+        const size_t row = (size_t)(first + min(t, n - 1));
+        const float kv = A.k[row * A.k_ld + A.k_off + kh * dim + k], qv = A.q[row * A.q_ld + A.q_off + qh * dim + k];
+        sk[t][k] = t < n ? kv : 0.f;
+        sq[t][k] = t < n ? qv : 0.f;
+    }
+    if (tid < DC) {
+        float la = 0.f, b = 0.f;
+        if (tid < n) {
+            const size_t row = (size_t)(first + tid);
+            la = -A.rate[h] * ds_softplus(A.step[row * A.step_ld + A.step_off + h] + A.step_bias[h]);
+            b = ds_sigmoid(A.beta[row * A.beta_ld + A.beta_off + h]);
+        }
+        lg[tid] = la;
+        sb[tid] = b;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        float sum = 0.f;
+        for (int t = 0; t < DC; ++t) {
+            sum += lg[t];
+            lg[t] = sum;
+        }
+    }
+    __syncthreads();
+    const size_t at = ((size_t)blockIdx.x * heads + h);
+    float* T_out = A.chunk_state + at * (2 * DC * DC);
+    float* M_out = T_out + DC * DC;
+    for (int i = tid; i < DC * DC; i += 256) {
+        const int t = i / DC, j = i - t * DC;
+        float kk = 0.f, qk = 0.f;
+        if (j <= t) {
+            for (int k = 0; k < dim; ++k) {
+                kk = fmaf(sk[t][k], sk[j][k], kk);
+                qk = fmaf(sq[t][k], sk[j][k], qk);
+            }
+            const float w = expf(lg[t] - lg[j]);
+            kk *= w * sb[t];
+            qk *= w;
+        }
+        sL[t][j] = j < t ? kk : 0.f;
+        M_out[i] = qk;
+    }
+    __syncthreads();
+    if (tid < DC) {
+        // column tid of (I + L)^-1 by forward substitution, then times b of that column
+        float x[DC];
+#pragma unroll
+        for (int t = 0; t < DC; ++t) {
+            float acc = t == tid ? 1.f : 0.f;
+#pragma unroll
+            for (int j = 0; j < t; ++j) acc = fmaf(-sL[t][j], x[j], acc);
+            x[t] = acc;
+        }
+        const float b = sb[tid];
+#pragma unroll
+        for (int t = 0; t < DC; ++t) T_out[t * DC + tid] = x[t] * b;
+        A.chunk_decay[at * DC + tid] = lg[tid];
+    }
+}
+
+__global__ __launch_bounds__(256) void k_delta_chunk_scan(const DecayScanArgs A) {
+    __shared__ float sS[DMAXK][DVB], sk[DC][DMAXK + 1], sq[DC][DMAXK + 1], sU[DC][DVB], sT[DC][DC], sM[DC][DC];
+    __shared__ float sg[DC], sw[DC];
+    float (*sR)[DVB] = reinterpret_cast<float (*)[DVB]>(&sq[0][0]);      // R lies where Q lay, once Q has been used
+    const int r = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * DVB;
+    const int tid = threadIdx.x, v = tid % DVB, g = tid / DVB;            // g: 0 .. 7
+    constexpr int TPT = DC / 8;                                             // tokens of a chunk a thread takes
+    const int heads = A.heads, dim = A.dim, vdim = A.vdim;
+    const bool live = v0 + v < vdim;
+    const int n_all = A.seg_len[r], n_chunks = (n_all + DC - 1) / DC;
+    const int qh = h / A.q_div, kh = h / A.k_div;
+    float* S_at = A.state + (((size_t)A.slot[r] * heads + h) * dim) * vdim;
+    for (int i = tid; i < dim * DVB; i += 256) {
+        const int k = i / DVB, c = i - k * DVB;
+        sS[k][c] = (v0 + c) < vdim ? S_at[(size_t)k * vdim + v0 + c] : 0.f;
+    }
+    const int kpt = (dim + 7) / 8;
+    for (int chunk = 0; chunk < n_chunks; ++chunk) {
+        const int first = A.seg_start[r] + chunk * DC, n = min(DC, n_all - chunk * DC);
+        const size_t at = ((size_t)(r * A.max_chunks + chunk) * heads + h);
+        const float* T_in = A.chunk_state + at * (2 * DC * DC);
+        const float* M_in = T_in + DC * DC;
+        __syncthreads();                                 // the chunk before has been used, the state is whole
+        for (int i = tid; i < DC * dim; i += 256) {
+            const int t = i / dim, k = i - t * dim;
+            const size_t row = (size_t)(first + min(t, n - 1));
+            const float kv = A.k[row * A.k_ld + A.k_off + kh * dim + k], qv = A.q[row * A.q_ld + A.q_off + qh * dim + k];
+            sk[t][k] = t < n ? kv : 0.f;
+            sq[t][k] = t < n ? qv : 0.f;
+        }
+        for (int i = tid; i < DC * DC; i += 256) {
+            sT[i / DC][i % DC] = T_in[i];
+            sM[i / DC][i % DC] = M_in[i];
+        }
+        if (tid < DC) {
+            const float l = A.chunk_decay[at * DC + tid], last = A.chunk_decay[at * DC + DC - 1];
+            sg[tid] = expf(l);
+            sw[tid] = expf(last - l);
+        }
+        float vt[TPT];
+#pragma unroll
+        for (int i = 0; i < TPT; ++i) {
+            const int t = g + 8 * i;
+            vt[i] = (t < n && live) ? A.v[(size_t)(first + t) * A.v_ld + A.v_off + h * vdim + v0 + v] : 0.f;
+        }
+        __syncthreads();
+        // what the state says of the chunk's keys and queries
+        float p[TPT], s[TPT];
+#pragma unroll
+        for (int i = 0; i < TPT; ++i) p[i] = s[i] = 0.f;
+        for (int k = 0; k < dim; ++k) {
+            const float sv = sS[k][v];
+#pragma unroll
+            for (int i = 0; i < TPT; ++i) {
+                p[i] = fmaf(sk[g + 8 * i][k], sv, p[i]);
+                s[i] = fmaf(sq[g + 8 * i][k], sv, s[i]);
+            }
+        }
+        __syncthreads();                                 // Q has been used: R goes where it lay
+#pragma unroll
+        for (int i = 0; i < TPT; ++i) {
+            const int t = g + 8 * i;
+            sR[t][v] = vt[i] - sg[t] * p[i];
+            s[i] *= sg[t];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < TPT; ++i) {
+            const int t = g + 8 * i;
+            float acc = 0.f;
+            for (int j = 0; j <= t; ++j) acc = fmaf(sT[t][j], sR[j][v], acc);
+            sU[t][v] = acc;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < TPT; ++i) {
+            const int t = g + 8 * i;
+            float acc = s[i];
+            for (int j = 0; j <= t; ++j) acc = fmaf(sM[t][j], sU[j][v], acc);
+            if (t < n && live) A.out[(size_t)(first + t) * heads * vdim + (size_t)h * vdim + v0 + v] = acc;
+        }
+        // the state behind the chunk: this thread's rows of its column
+        const float g_last = sg[DC - 1];
+        for (int m = 0; m < kpt; ++m) {
+            const int k = g * kpt + m;
+            if (k < dim) {
+                float acc = g_last * sS[k][v];
+                for (int j = 0; j < DC; ++j) acc = fmaf(sw[j] * sk[j][k], sU[j][v], acc);
+                sS[k][v] = acc;
+            }
+        }
+    }
+    __syncthreads();
+    for (int i = tid; i < dim * DVB; i += 256) {
+        const int k = i / DVB, c = i - k * DVB;
+        if (v0 + c < vdim) S_at[(size_t)k * vdim + v0 + c] = sS[k][c];
+    }
+}
+
+extern "C" int imparo_delta_chunk_tokens() { return DC; }
+extern "C" int imparo_delta_chunk_max_dim() { return DMAXK; }
+
 extern "C" int imparo_decay_scan(const float* q, int q_ld, int q_off, int q_div, const float* k, int k_ld, int k_off,
                                  int k_div, const float* v, int v_ld, int v_off, const float* decay_const,
                                  const float* step, int step_ld, int step_off, const float* step_bias,
@@ -198,7 +386,8 @@ extern "C" int imparo_decay_scan(const float* q, int q_ld, int q_off, int q_div,
     if (!decay_const && (!step || !step_bias || !rate)) return IMPARO_BAD_ARGUMENT;
     if (v_times_step && decay_const) return IMPARO_BAD_ARGUMENT;
     if (chunk_tokens < 0 || chunk_tokens % DS_TOKENS) return IMPARO_BAD_ARGUMENT;
-    if (chunk_tokens && (beta || max_chunks < 1 || !chunk_state || !chunk_decay)) return IMPARO_BAD_ARGUMENT;
+    if (chunk_tokens && (max_chunks < 1 || !chunk_state || !chunk_decay)) return IMPARO_BAD_ARGUMENT;
+    if (chunk_tokens && beta && (chunk_tokens != DC || dim > DMAXK || decay_const)) return IMPARO_BAD_ARGUMENT;
     if (n_rows < 0 || heads < 1 || dim < 1 || dim > DS_MAX_DIM || vdim < 1) return IMPARO_BAD_ARGUMENT;
     if (q_div < 1 || k_div < 1 || heads % q_div || heads % k_div) return IMPARO_BAD_ARGUMENT;
     if (q_off < 0 || k_off < 0 || v_off < 0 || q_ld < q_off + heads / q_div * dim || k_ld < k_off + heads / k_div * dim ||
@@ -222,6 +411,13 @@ extern "C" int imparo_decay_scan(const float* q, int q_ld, int q_off, int q_div,
                              step, step_ld, step_off, step_bias, rate, v_times_step, beta, beta_ld, beta_off, skip,
                              state, seg_start, seg_len, slot, out, heads, dim, vdim, kpt,
                              chunk_tokens, max_chunks, chunk_state, chunk_decay};
+    if (beta && chunk_tokens) {
+        // the delta rule in chunks: chunk_state holds T and M of every chunk, chunk_decay the logarithms of its decays
+        if (v_times_step || skip) return IMPARO_BAD_ARGUMENT;
+        k_delta_chunk_prepare<<<dim3(n_rows * max_chunks, heads), 256, 0, s>>>(args);
+        k_delta_chunk_scan<<<dim3(n_rows, heads, (vdim + DVB - 1) / DVB), 256, 0, s>>>(args);
+        return launch_status();
+    }
 #define DS_LAUNCH(KS)                                                                                                \
     if (beta) {                                                                                                      \
         k_decay_scan<KS, 0, true><<<grid, threads, 0, s>>>(args);                                                    \

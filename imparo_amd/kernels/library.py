@@ -85,6 +85,8 @@ _SIGNATURES = {
     # chunk_decay, stream
     "imparo_decay_scan": [P, I, I, I, P, I, I, I, P, I, I, P, P, I, I, P, P, I, P, I, I, P, P, P, P, P, P, I, I, I, I, I, I,
                           P, P, P],
+    "imparo_delta_chunk_tokens": [],
+    "imparo_delta_chunk_max_dim": [],
     "imparo_head_prepare": [P, I, I, I, I, I, I, F, P, I, I, P, I, F, F, P],
     "imparo_gated_group_norm": [P, P, I, I, P, P, I, I, I, I, F, I, P],
     "imparo_clamped_glu": [P, P, I, I, I, I, F, F, P],

@@ -1138,12 +1138,26 @@ DECAY_SCAN_MAX_DIM = 512          # state rows a head
 DECAY_SCAN_CHUNK = 64             # tokens a chunk when a long segment's chunks run side by side
 
 
-def decay_scan_chunks(max_seg_len: int, delta: bool = False):
-    """(chunk_tokens, max_chunks) for `decay_scan`: (0, 1) for one launch, which short segments and the delta
-    rule take; else chunks of DECAY_SCAN_CHUNK tokens, as many as the longest segment makes."""
-    if delta or max_seg_len < 4 * DECAY_SCAN_CHUNK:
+def decay_scan_chunks(max_seg_len: int, delta: bool = False, dim: int = 0):
+    """(chunk_tokens, max_chunks) for `decay_scan`: (0, 1) for one launch, which short segments take; else chunks
+    of DECAY_SCAN_CHUNK tokens (the delta rule: of its own chunk size, for heads of up to its largest dim), as
+    many as the longest segment makes."""
+    if delta:
+        chunk = int(library().imparo_delta_chunk_tokens())
+        if max_seg_len < 2 * chunk or dim > int(library().imparo_delta_chunk_max_dim()):
+            return 0, 1
+        return chunk, -(-int(max_seg_len) // chunk)
+    if max_seg_len < 4 * DECAY_SCAN_CHUNK:
         return 0, 1
     return DECAY_SCAN_CHUNK, -(-int(max_seg_len) // DECAY_SCAN_CHUNK)
+
+
+def decay_scan_scratch(n_rows: int, max_chunks: int, heads: int, dim: int, vdim: int, delta: bool = False):
+    """Floats of (chunk_state, chunk_decay) that `decay_scan` needs when it walks in chunks."""
+    if delta:
+        chunk = int(library().imparo_delta_chunk_tokens())
+        return n_rows * max_chunks * heads * 2 * chunk * chunk, n_rows * max_chunks * heads * chunk
+    return n_rows * max_chunks * heads * dim * vdim, n_rows * max_chunks * heads
 
 
 def decay_scan(q: torch.Tensor, q_off: int, q_div: int, k: torch.Tensor, k_off: int, k_div: int, v: torch.Tensor,
@@ -1169,9 +1183,7 @@ def decay_scan(q: torch.Tensor, q_off: int, q_div: int, k: torch.Tensor, k_off: 
     if (decay_const is None) == (step is None):
         raise KernelArgumentError("decay_scan: the decay is a constant a head or comes from projected steps")
     if chunk_tokens:
-        if beta is not None:
-            raise KernelArgumentError("decay_scan: the delta rule is walked in one launch")
-        need_s, need_d = n_rows * max_chunks * heads * dim * vdim, n_rows * max_chunks * heads
+        need_s, need_d = decay_scan_scratch(n_rows, max_chunks, heads, dim, vdim, beta is not None)
         if chunk_state is None or chunk_decay is None or chunk_state.numel() < need_s or chunk_decay.numel() < need_d:
             raise KernelArgumentError("decay_scan: the scratch for the chunks' states is too small")
     _check(library().imparo_decay_scan(

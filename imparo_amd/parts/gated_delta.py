@@ -116,9 +116,17 @@ class GatedDelta:
         # q and k heads as unit vectors; the queries carry dim^(-1/2)
         ops.head_prepare(qkv, 0, 2 * Hk, dk, unit=True, unit_eps=UNIT_EPS, n_first=Hk, scale_first=float(dk) ** -0.5)
         o = ctx.workspace.get("delta_o", (T, H * dv), torch.float32)
+        # a long portion: the rule in chunks (a triangle solved a chunk, side by side; then the chunks in order)
+        chunk_tokens, max_chunks = ops.decay_scan_chunks(ctx.max_seg_len, delta=True, dim=dk)
+        chunk_state = chunk_decay = None
+        if chunk_tokens:
+            n_state, n_decay = ops.decay_scan_scratch(ctx.n_rows, max_chunks, H, dk, dv, delta=True)
+            chunk_state = ctx.workspace.get("scan_chunk_state", (n_state,), torch.float32)
+            chunk_decay = ctx.workspace.get("scan_chunk_decay", (n_decay,), torch.float32)
         ops.decay_scan(qkv, 0, H // Hk, qkv, Hk * dk, H // Hk, qkv, 2 * Hk * dk, state["state"], ctx.seg_start,
                        ctx.seg_len, ctx.slot, o, H, dk, dv, step=rows, step_off=C + H, step_bias=self.dt_bias,
-                       rate=self.rate, beta=rows, beta_off=C)
+                       rate=self.rate, beta=rows, beta_off=C, chunk_tokens=chunk_tokens, max_chunks=max_chunks,
+                       chunk_state=chunk_state, chunk_decay=chunk_decay)
         gated = ctx.workspace.get("delta_gated", (T, H * dv), self.out.in_dtype, alias="mixer_mid")
         ops.gated_group_norm(o, rows, C + 2 * H, self.norm, H, self.eps, gated, gate_first=False)
         return self.out(ctx, gated, torch.float32, "mixer_out", sliced_ok=True, into=ctx.stream)

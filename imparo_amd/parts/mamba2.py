@@ -116,8 +116,9 @@ class Mamba2:
         chunk_tokens, max_chunks = ops.decay_scan_chunks(ctx.max_seg_len)
         chunk_state = chunk_decay = None
         if chunk_tokens:
-            chunk_state = ctx.workspace.get("scan_chunk_state", (ctx.n_rows * max_chunks * H * N * P,), torch.float32)
-            chunk_decay = ctx.workspace.get("scan_chunk_decay", (ctx.n_rows * max_chunks * H,), torch.float32)
+            n_state, n_decay = ops.decay_scan_scratch(ctx.n_rows, max_chunks, H, N, P)
+            chunk_state = ctx.workspace.get("scan_chunk_state", (n_state,), torch.float32)
+            chunk_decay = ctx.workspace.get("scan_chunk_decay", (n_decay,), torch.float32)
         ops.decay_scan(xbc, inner + G * N, H // G, xbc, inner, H // G, xbc, 0, state["state"], ctx.seg_start, ctx.seg_len,
                        ctx.slot, y, H, N, P, step=rows, step_off=inner + C, step_bias=self.dt_bias, rate=self.rate,
                        v_times_step=True, skip=self.D, chunk_tokens=chunk_tokens, max_chunks=max_chunks,

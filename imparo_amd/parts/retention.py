@@ -95,8 +95,9 @@ class Retention:
         chunk_tokens, max_chunks = ops.decay_scan_chunks(ctx.max_seg_len)
         chunk_state = chunk_decay = None
         if chunk_tokens:
-            chunk_state = ctx.workspace.get("scan_chunk_state", (ctx.n_rows * max_chunks * H * d * dv,), torch.float32)
-            chunk_decay = ctx.workspace.get("scan_chunk_decay", (ctx.n_rows * max_chunks * H,), torch.float32)
+            n_state, n_decay = ops.decay_scan_scratch(ctx.n_rows, max_chunks, H, d, dv)
+            chunk_state = ctx.workspace.get("scan_chunk_state", (n_state,), torch.float32)
+            chunk_decay = ctx.workspace.get("scan_chunk_decay", (n_decay,), torch.float32)
         ops.decay_scan(rows, 0, 1, rows, H * d, 1, rows, 2 * H * d, ctx.fixed_arrays(site)["state"], ctx.seg_start,
                        ctx.seg_len, ctx.slot, o, H, d, dv, decay_const=self.decay, chunk_tokens=chunk_tokens,
                        max_chunks=max_chunks, chunk_state=chunk_state, chunk_decay=chunk_decay)

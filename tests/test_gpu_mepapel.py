@@ -126,13 +126,14 @@ def plain_scan(q, k, v, a, beta, S):
                                           (1, 1, 200, 300), (2, 1, 512, 8), (6, 3, 64, 128)])
 def test_recurrence_kernel_continues_over_segments_in_used_slots(H, share, d, dv, kind):
     """Three requests in slots that held something else, fed in segments of changing length (one token, two, a long
-    one that the kernel walks in chunks side by side): results and states are those of one walk over all tokens.
+    one that the kernel walks in chunks: side by side where the decay is plain, a triangle solved a chunk for the
+    delta rule): results and states are those of one walk over all tokens.
     Heads share queries and keys in groups of `share`; `steps` also multiplies the values by the step and adds the
     skip, as a state-space layer does."""
     from imparo_amd.kernels import ops
     g = torch.Generator().manual_seed(H * 1000 + d + dv)
-    lens, slots, n_slots = [341, 7, 64], [5, 0, 3], 6
-    cuts = [[1, 2, 300, 38], [7], [5, 1, 1, 57]]
+    lens, slots, n_slots = [341, 7, 107], [5, 0, 3], 6
+    cuts = [[1, 2, 300, 38], [7], [5, 1, 70, 31]]
     Hs = H // share
     f64 = torch.float64
     data = []
@@ -173,11 +174,11 @@ def test_recurrence_kernel_continues_over_segments_in_used_slots(H, share, d, dv
         T = rows_t.shape[0]
         starts = np.cumsum([0] + seg[:-1])
         out = torch.full((T, H * dv), 7.0, device=DEV)
-        chunk_tokens, max_chunks = ops.decay_scan_chunks(max(seg), delta=kind == "delta")
+        chunk_tokens, max_chunks = ops.decay_scan_chunks(max(seg), delta=kind == "delta", dim=d)
         cs = cd = None
         if chunk_tokens:
-            cs = torch.empty(len(rows) * max_chunks * H * d * dv, device=DEV)
-            cd = torch.empty(len(rows) * max_chunks * H, device=DEV)
+            n_state, n_decay = ops.decay_scan_scratch(len(rows), max_chunks, H, d, dv, delta=kind == "delta")
+            cs, cd = torch.empty(n_state, device=DEV), torch.empty(n_decay, device=DEV)
         kw = dict(decay_const=dev(const)) if kind == "constant" else dict(
             step=rows_t, step_off=2 * Hs * d + H * dv, step_bias=dev(bias), rate=dev(rate))
         if kind == "steps":
