@@ -272,101 +272,166 @@ __global__ __launch_bounds__(256) void k_delta_chunk_prepare(const DecayScanArgs
     }
 }
 
+// What a block of the walk asks of memory for one chunk, in registers: asked for while the chunk before is worked on.
+#define DPIECES (DC * DMAXK / 256)        // elements of a chunk's K (and Q) a thread brings at most
+struct DeltaFetch {
+    float k[DPIECES], q[DPIECES], t[DC * DC / 256], m[DC * DC / 256], v[DC / 8], l, last;
+};
+
+template <int VB>
 __global__ __launch_bounds__(256) void k_delta_chunk_scan(const DecayScanArgs A) {
-    __shared__ float sS[DMAXK][DVB], sk[DC][DMAXK + 1], sq[DC][DMAXK + 1], sU[DC][DVB], sT[DC][DC], sM[DC][DC];
-    __shared__ float sg[DC], sw[DC];
-    float (*sR)[DVB] = reinterpret_cast<float (*)[DVB]>(&sq[0][0]);      // R lies where Q lay, once Q has been used
-    const int r = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * DVB;
-    const int tid = threadIdx.x, v = tid % DVB, g = tid / DVB;            // g: 0 .. 7
-    constexpr int TPT = DC / 8;                                             // tokens of a chunk a thread takes
+    constexpr int KLD = DMAXK + 4;                       // floats between two tokens' rows: whole 16-byte pieces
+    constexpr int NG = 256 / VB;                         // threads a value column: each takes every NG-th token
+    constexpr int TPT = DC / NG;                         // tokens of a chunk a thread takes
+    constexpr int KPT = DMAXK / NG;                      // state rows of its column a thread takes at most
+    __shared__ __attribute__((aligned(16))) float sk[DC][KLD], sq[DC][KLD];
+    __shared__ float sS[DMAXK][VB], sU[DC][VB], sT[DC][DC], sM[DC][DC], sg[DC], sw[DC];
+    float (*sR)[VB] = reinterpret_cast<float (*)[VB]>(&sq[0][0]);        // R lies where Q lay, once Q has been used
+    const int r = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * VB;
+    const int tid = threadIdx.x, v = tid % VB, g = tid / VB;
     const int heads = A.heads, dim = A.dim, vdim = A.vdim;
+    const int dim4 = (dim + 3) & ~3;
     const bool live = v0 + v < vdim;
     const int n_all = A.seg_len[r], n_chunks = (n_all + DC - 1) / DC;
     const int qh = h / A.q_div, kh = h / A.k_div;
     float* S_at = A.state + (((size_t)A.slot[r] * heads + h) * dim) * vdim;
-    for (int i = tid; i < dim * DVB; i += 256) {
-        const int k = i / DVB, c = i - k * DVB;
-        sS[k][c] = (v0 + c) < vdim ? S_at[(size_t)k * vdim + v0 + c] : 0.f;
+    for (int i = tid; i < dim4 * VB; i += 256) {
+        const int k = i / VB, c = i - k * VB;
+        sS[k][c] = (k < dim && (v0 + c) < vdim) ? S_at[(size_t)k * vdim + v0 + c] : 0.f;
     }
-    const int kpt = (dim + 7) / 8;
-    for (int chunk = 0; chunk < n_chunks; ++chunk) {
+    // which (token, state row) of a chunk's K and Q this thread brings: the same for every chunk
+    int piece_t[DPIECES];
+#pragma unroll
+    for (int it = 0; it < DPIECES; ++it) piece_t[it] = min((tid + 256 * it) / dim4, DC - 1);
+    DeltaFetch f;
+    // every address is clamped into the segment (no load under a branch); what lies beyond is zeroed when it is used
+    auto fetch = [&](int chunk) {
         const int first = A.seg_start[r] + chunk * DC, n = min(DC, n_all - chunk * DC);
         const size_t at = ((size_t)(r * A.max_chunks + chunk) * heads + h);
         const float* T_in = A.chunk_state + at * (2 * DC * DC);
-        const float* M_in = T_in + DC * DC;
-        __syncthreads();                                 // the chunk before has been used, the state is whole
-        for (int i = tid; i < DC * dim; i += 256) {
-            const int t = i / dim, k = i - t * dim;
+#pragma unroll
+        for (int it = 0; it < DPIECES; ++it) {
+            const int t = piece_t[it], k = min(max(tid + 256 * it - t * dim4, 0), dim - 1);
             const size_t row = (size_t)(first + min(t, n - 1));
-            const float kv = A.k[row * A.k_ld + A.k_off + kh * dim + k], qv = A.q[row * A.q_ld + A.q_off + qh * dim + k];
-            sk[t][k] = t < n ? kv : 0.f;
-            sq[t][k] = t < n ? qv : 0.f;
+            f.k[it] = A.k[row * A.k_ld + A.k_off + kh * dim + k];
+            f.q[it] = A.q[row * A.q_ld + A.q_off + qh * dim + k];
         }
-        for (int i = tid; i < DC * DC; i += 256) {
-            sT[i / DC][i % DC] = T_in[i];
-            sM[i / DC][i % DC] = M_in[i];
+#pragma unroll
+        for (int it = 0; it < DC * DC / 256; ++it) {
+            f.t[it] = T_in[tid + 256 * it];
+            f.m[it] = T_in[DC * DC + tid + 256 * it];
+        }
+        f.l = A.chunk_decay[at * DC + (tid & (DC - 1))];
+        f.last = A.chunk_decay[at * DC + DC - 1];
+#pragma unroll
+        for (int i = 0; i < TPT; ++i) {
+            const int t = min(g + NG * i, n - 1);
+            f.v[i] = A.v[(size_t)(first + t) * A.v_ld + A.v_off + h * vdim + min(v0 + v, vdim - 1)];
+        }
+    };
+    fetch(0);
+    const int kpt = (((dim4 + NG - 1) / NG) + 3) & ~3;   // this thread's state rows: kpt from g * kpt on
+    for (int chunk = 0; chunk < n_chunks; ++chunk) {
+        const int first = A.seg_start[r] + chunk * DC, n = min(DC, n_all - chunk * DC);
+        __syncthreads();                                 // the chunk before has been used, the state is whole
+#pragma unroll
+        for (int it = 0; it < DPIECES; ++it) {
+            const int i = tid + 256 * it, t = piece_t[it], k = i - t * dim4;
+            if (i < DC * dim4) {
+                const bool on = t < n && k < dim;
+                sk[t][k] = on ? f.k[it] : 0.f;
+                sq[t][k] = on ? f.q[it] : 0.f;
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < DC * DC / 256; ++it) {
+            const int i = tid + 256 * it;
+            sT[i / DC][i % DC] = f.t[it];
+            sM[i / DC][i % DC] = f.m[it];
         }
         if (tid < DC) {
-            const float l = A.chunk_decay[at * DC + tid], last = A.chunk_decay[at * DC + DC - 1];
-            sg[tid] = expf(l);
-            sw[tid] = expf(last - l);
+            sg[tid] = expf(f.l);
+            sw[tid] = expf(f.last - f.l);
         }
         float vt[TPT];
 #pragma unroll
-        for (int i = 0; i < TPT; ++i) {
-            const int t = g + 8 * i;
-            vt[i] = (t < n && live) ? A.v[(size_t)(first + t) * A.v_ld + A.v_off + h * vdim + v0 + v] : 0.f;
-        }
+        for (int i = 0; i < TPT; ++i) vt[i] = (g + NG * i < n && live) ? f.v[i] : 0.f;
         __syncthreads();
+        fetch(min(chunk + 1, n_chunks - 1));             // on its way while this chunk is worked on (no load under a branch)
         // what the state says of the chunk's keys and queries
         float p[TPT], s[TPT];
 #pragma unroll
         for (int i = 0; i < TPT; ++i) p[i] = s[i] = 0.f;
-        for (int k = 0; k < dim; ++k) {
-            const float sv = sS[k][v];
+#pragma unroll 4
+        for (int k = 0; k < dim4; k += 4) {
+            const float s0 = sS[k][v], s1 = sS[k + 1][v], s2 = sS[k + 2][v], s3 = sS[k + 3][v];
 #pragma unroll
             for (int i = 0; i < TPT; ++i) {
-                p[i] = fmaf(sk[g + 8 * i][k], sv, p[i]);
-                s[i] = fmaf(sq[g + 8 * i][k], sv, s[i]);
+                const float4 kk = *reinterpret_cast<const float4*>(&sk[g + NG * i][k]);
+                const float4 qq = *reinterpret_cast<const float4*>(&sq[g + NG * i][k]);
+                p[i] = fmaf(kk.w, s3, fmaf(kk.z, s2, fmaf(kk.y, s1, fmaf(kk.x, s0, p[i]))));
+                s[i] = fmaf(qq.w, s3, fmaf(qq.z, s2, fmaf(qq.y, s1, fmaf(qq.x, s0, s[i]))));
             }
         }
-        __syncthreads();                                 // Q has been used: R goes where it lay
+        __syncthreads();                                 // K and Q have been used: R goes where Q lay, K takes its weights
 #pragma unroll
         for (int i = 0; i < TPT; ++i) {
-            const int t = g + 8 * i;
+            const int t = g + NG * i;
             sR[t][v] = vt[i] - sg[t] * p[i];
             s[i] *= sg[t];
         }
+        for (int i = tid; i < DC * dim4; i += 256) sk[i / dim4][i % dim4] *= sw[i / dim4];
         __syncthreads();
+        // (T and M are zero above their diagonals: the sums run over the whole chunk, so that the reads of
+        // several steps can be under way at once; a product with zero adds nothing)
+        float u[TPT];
 #pragma unroll
-        for (int i = 0; i < TPT; ++i) {
-            const int t = g + 8 * i;
-            float acc = 0.f;
-            for (int j = 0; j <= t; ++j) acc = fmaf(sT[t][j], sR[j][v], acc);
-            sU[t][v] = acc;
+        for (int i = 0; i < TPT; ++i) u[i] = 0.f;
+#pragma unroll 8
+        for (int j = 0; j < DC; ++j) {
+            const float rv = sR[j][v];
+#pragma unroll
+            for (int i = 0; i < TPT; ++i) u[i] = fmaf(sT[g + NG * i][j], rv, u[i]);
         }
+#pragma unroll
+        for (int i = 0; i < TPT; ++i) sU[g + NG * i][v] = u[i];
         __syncthreads();
+#pragma unroll 8
+        for (int j = 0; j < DC; ++j) {
+            const float uv = sU[j][v];
+#pragma unroll
+            for (int i = 0; i < TPT; ++i) s[i] = fmaf(sM[g + NG * i][j], uv, s[i]);
+        }
 #pragma unroll
         for (int i = 0; i < TPT; ++i) {
-            const int t = g + 8 * i;
-            float acc = s[i];
-            for (int j = 0; j <= t; ++j) acc = fmaf(sM[t][j], sU[j][v], acc);
-            if (t < n && live) A.out[(size_t)(first + t) * heads * vdim + (size_t)h * vdim + v0 + v] = acc;
+            const int t = g + NG * i;
+            if (t < n && live) A.out[(size_t)(first + t) * heads * vdim + (size_t)h * vdim + v0 + v] = s[i];
         }
         // the state behind the chunk: this thread's rows of its column
         const float g_last = sg[DC - 1];
-        for (int m = 0; m < kpt; ++m) {
-            const int k = g * kpt + m;
-            if (k < dim) {
-                float acc = g_last * sS[k][v];
-                for (int j = 0; j < DC; ++j) acc = fmaf(sw[j] * sk[j][k], sU[j][v], acc);
-                sS[k][v] = acc;
-            }
+        float acc[KPT];
+#pragma unroll
+        for (int m = 0; m < KPT; ++m) acc[m] = (m < kpt && g * kpt + m < dim4) ? g_last * sS[g * kpt + m][v] : 0.f;
+#pragma unroll 4
+        for (int j = 0; j < DC; ++j) {
+            const float u = sU[j][v];
+#pragma unroll
+            for (int m = 0; m < KPT; m += 4)
+                if (m < kpt && g * kpt + m < dim4) {
+                    const float4 w = *reinterpret_cast<const float4*>(&sk[j][g * kpt + m]);
+                    acc[m] = fmaf(w.x, u, acc[m]);
+                    acc[m + 1] = fmaf(w.y, u, acc[m + 1]);
+                    acc[m + 2] = fmaf(w.z, u, acc[m + 2]);
+                    acc[m + 3] = fmaf(w.w, u, acc[m + 3]);
+                }
         }
+#pragma unroll
+        for (int m = 0; m < KPT; ++m)
+            if (m < kpt && g * kpt + m < dim4) sS[g * kpt + m][v] = acc[m];
     }
     __syncthreads();
-    for (int i = tid; i < dim * DVB; i += 256) {
-        const int k = i / DVB, c = i - k * DVB;
+    for (int i = tid; i < dim * VB; i += 256) {
+        const int k = i / VB, c = i - k * VB;
         if (v0 + c < vdim) S_at[(size_t)k * vdim + v0 + c] = sS[k][c];
     }
 }
@@ -415,7 +480,11 @@ extern "C" int imparo_decay_scan(const float* q, int q_ld, int q_off, int q_div,
         // the delta rule in chunks: chunk_state holds T and M of every chunk, chunk_decay the logarithms of its decays
         if (v_times_step || skip) return IMPARO_BAD_ARGUMENT;
         k_delta_chunk_prepare<<<dim3(n_rows * max_chunks, heads), 256, 0, s>>>(args);
-        k_delta_chunk_scan<<<dim3(n_rows, heads, (vdim + DVB - 1) / DVB), 256, 0, s>>>(args);
+        // few blocks (a segment, few heads): narrower runs of columns make more of them
+        if ((long long)n_rows * heads * ((vdim + DVB - 1) / DVB) >= 256 || vdim <= 16)
+            k_delta_chunk_scan<DVB><<<dim3(n_rows, heads, (vdim + DVB - 1) / DVB), 256, 0, s>>>(args);
+        else
+            k_delta_chunk_scan<16><<<dim3(n_rows, heads, (vdim + 15) / 16), 256, 0, s>>>(args);
         return launch_status();
     }
 #define DS_LAUNCH(KS)                                                                                                \
