@@ -54,9 +54,11 @@ struct DecayScanArgs {
 // MODE 1: a chunk that is not the segment's last, from a zero state: its end state goes to chunk_state, the
 // product of its decays to chunk_decay, no results; MODE 2: a chunk from the state chunk_state holds for it,
 // with results; the last chunk writes the request's state.
-template <int KS, int MODE, bool DELTA>
+// V4: a thread's slice is whole 16-byte pieces, read as such.
+template <int KS, int MODE, bool DELTA, bool V4>
 __global__ __launch_bounds__(DS_MAX_THREADS) void k_decay_scan(const DecayScanArgs A) {
-    __shared__ float sq[DS_TOKENS][DS_MAX_DIM], sk[DS_TOKENS][DS_MAX_DIM], sv[DS_TOKENS][DS_MAX_THREADS];
+    __shared__ __attribute__((aligned(16))) float sq[DS_TOKENS][DS_MAX_DIM], sk[DS_TOKENS][DS_MAX_DIM];
+    __shared__ float sv[DS_TOKENS][DS_MAX_THREADS];
     __shared__ float sa[DS_TOKENS], sb[DS_TOKENS], sdt[DS_TOKENS];
     const int VB = blockDim.x / KS;                      // value columns of a block
     const int r = MODE == 0 ? blockIdx.x : blockIdx.x / A.max_chunks;
@@ -119,13 +121,31 @@ __global__ __launch_bounds__(DS_MAX_THREADS) void k_decay_scan(const DecayScanAr
             const float raw = sv[tok][vl];
             float val = raw * sdt[tok];
             float acc = 0.f;
+            float kk[DS_KPT], qq[DS_KPT];
+            if constexpr (V4) {
+#pragma unroll
+                for (int j = 0; j < DS_KPT; j += 4)
+                    if (j < kpt) {
+                        const float4 k4 = *reinterpret_cast<const float4*>(&sk[tok][ks * kpt + j]);
+                        const float4 q4 = *reinterpret_cast<const float4*>(&sq[tok][ks * kpt + j]);
+                        kk[j] = k4.x, kk[j + 1] = k4.y, kk[j + 2] = k4.z, kk[j + 3] = k4.w;
+                        qq[j] = q4.x, qq[j + 1] = q4.y, qq[j + 2] = q4.z, qq[j + 3] = q4.w;
+                    }
+            } else {
+#pragma unroll
+                for (int j = 0; j < DS_KPT; ++j)
+                    if (j < kpt) {
+                        kk[j] = sk[tok][ks * kpt + j];
+                        qq[j] = sq[tok][ks * kpt + j];
+                    }
+            }
             if constexpr (DELTA) {
                 float seen = 0.f;
 #pragma unroll
                 for (int j = 0; j < DS_KPT; ++j)
                     if (j < kpt) {
                         S[j] *= a;
-                        seen = fmaf(S[j], sk[tok][ks * kpt + j], seen);
+                        seen = fmaf(S[j], kk[j], seen);
                     }
 #pragma unroll
                 for (int off = 1; off < KS; off <<= 1) seen += __shfl_xor(seen, off, WAVE);
@@ -133,15 +153,15 @@ __global__ __launch_bounds__(DS_MAX_THREADS) void k_decay_scan(const DecayScanAr
 #pragma unroll
                 for (int j = 0; j < DS_KPT; ++j)
                     if (j < kpt) {
-                        S[j] = fmaf(sk[tok][ks * kpt + j], val, S[j]);
-                        acc = fmaf(S[j], sq[tok][ks * kpt + j], acc);
+                        S[j] = fmaf(kk[j], val, S[j]);
+                        acc = fmaf(S[j], qq[j], acc);
                     }
             } else {
 #pragma unroll
                 for (int j = 0; j < DS_KPT; ++j)
                     if (j < kpt) {
-                        S[j] = fmaf(sk[tok][ks * kpt + j], val, a * S[j]);
-                        if constexpr (MODE != 1) acc = fmaf(S[j], sq[tok][ks * kpt + j], acc);
+                        S[j] = fmaf(kk[j], val, a * S[j]);
+                        if constexpr (MODE != 1) acc = fmaf(S[j], qq[j], acc);
                     }
                 if constexpr (MODE == 1) decay_all *= a;
             }
@@ -487,18 +507,23 @@ extern "C" int imparo_decay_scan(const float* q, int q_ld, int q_off, int q_div,
             k_delta_chunk_scan<16><<<dim3(n_rows, heads, (vdim + 15) / 16), 256, 0, s>>>(args);
         return launch_status();
     }
+#define DS_PASS(KS, MODE, DELTA)                                                                                     \
+    if (kpt % 4 == 0)                                                                                                \
+        k_decay_scan<KS, MODE, DELTA, true><<<grid, threads, 0, s>>>(args);                                         \
+    else                                                                                                             \
+        k_decay_scan<KS, MODE, DELTA, false><<<grid, threads, 0, s>>>(args)
 #define DS_LAUNCH(KS)                                                                                                \
     if (beta) {                                                                                                      \
-        k_decay_scan<KS, 0, true><<<grid, threads, 0, s>>>(args);                                                    \
+        DS_PASS(KS, 0, true);                                                                                        \
     } else if (!chunk_tokens) {                                                                                      \
-        k_decay_scan<KS, 0, false><<<grid, threads, 0, s>>>(args);                                                   \
+        DS_PASS(KS, 0, false);                                                                                       \
     } else {                                                                                                         \
-        k_decay_scan<KS, 1, false><<<grid, threads, 0, s>>>(args);                                                   \
+        DS_PASS(KS, 1, false);                                                                                       \
         const long long entries = (long long)n_rows * heads * dim * vdim;                                            \
         k_decay_carry<<<(unsigned)((entries + 255) / 256), 256, 0, s>>>(chunk_state, chunk_decay, state, seg_len,    \
                                                                         slot, n_rows, heads, dim, vdim,              \
                                                                         chunk_tokens, max_chunks);                   \
-        k_decay_scan<KS, 2, false><<<grid, threads, 0, s>>>(args);                                                   \
+        DS_PASS(KS, 2, false);                                                                                       \
     }
     switch (ks) {
         case 1: DS_LAUNCH(1); break;
@@ -510,6 +535,7 @@ extern "C" int imparo_decay_scan(const float* q, int q_ld, int q_off, int q_div,
         default: return IMPARO_BAD_ARGUMENT;
     }
 #undef DS_LAUNCH
+#undef DS_PASS
     return launch_status();
 }
 
