@@ -14,7 +14,8 @@
 //
 // A long segment of the first form is walked in three launches, its chunks side by side (the recurrence
 // is linear in S with a scalar factor: after a chunk S = (product of the chunk's a) S_before + what the chunk
-// makes of a zero state). The delta rule's transition is a matrix (a (I - b k k^T)), so it is walked in one.
+// makes of a zero state). The delta rule's transition is a matrix (a (I - b k k^T)): its long segments take the
+// form in chunks further down (a triangle solved a chunk, then the chunks in order), short ones this walk.
 //
 // Beside it: what such mixers do to a head before the walk (unit length, rotation, a factor) and to the
 // heads behind it (a gate and a norm in groups of the row).
@@ -501,10 +502,14 @@ extern "C" int imparo_decay_scan(const float* q, int q_ld, int q_off, int q_div,
         if (v_times_step || skip) return IMPARO_BAD_ARGUMENT;
         k_delta_chunk_prepare<<<dim3(n_rows * max_chunks, heads), 256, 0, s>>>(args);
         // few blocks (a segment, few heads): narrower runs of columns make more of them
-        if ((long long)n_rows * heads * ((vdim + DVB - 1) / DVB) >= 256 || vdim <= 16)
+        // (a column's arithmetic is the same whatever the width of its run: the same bits)
+        const long long rh = (long long)n_rows * heads;
+        if (rh * ((vdim + DVB - 1) / DVB) >= 256 || vdim <= 8)
             k_delta_chunk_scan<DVB><<<dim3(n_rows, heads, (vdim + DVB - 1) / DVB), 256, 0, s>>>(args);
-        else
+        else if (rh * ((vdim + 15) / 16) >= 256 || vdim <= 8)
             k_delta_chunk_scan<16><<<dim3(n_rows, heads, (vdim + 15) / 16), 256, 0, s>>>(args);
+        else
+            k_delta_chunk_scan<8><<<dim3(n_rows, heads, (vdim + 7) / 8), 256, 0, s>>>(args);
         return launch_status();
     }
 #define DS_PASS(KS, MODE, DELTA)                                                                                     \
