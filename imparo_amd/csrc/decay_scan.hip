@@ -617,6 +617,7 @@ __global__ __launch_bounds__(256) void k_gated_group_norm(const float* __restric
     const float* xr = x + (size_t)t * width + (size_t)g * part;
     const float* gr = gate ? gate + (size_t)t * gate_ld + gate_off + (size_t)g * part : nullptr;
     float ss = 0.f;
+#pragma unroll 4
     for (int i = first; i < part; i += stride) {
         float y = xr[i];
         if (gate_first && gr) y *= ds_silu(gr[i]);
@@ -624,6 +625,7 @@ __global__ __launch_bounds__(256) void k_gated_group_norm(const float* __restric
     }
     ss = WHOLE_BLOCK ? block_sum(ss, scratch) : wave_sum(ss);
     const float rs = 1.0f / sqrtf(ss / (float)part + eps);
+#pragma unroll 4
     for (int i = first; i < part; i += stride) {
         float y = xr[i];
         const float gv = gr ? ds_silu(gr[i]) : 1.f;
@@ -693,39 +695,58 @@ extern "C" int imparo_clamped_glu(const float* gu, void* out, int out_dtype, int
 // ---------------------------------------------------------------- sums of mixers and of experts
 // out[t, c] (+)= sum_i f_i * rms_norm(a_i[t])[c] * w_i[c] over up to two inputs (each maybe in slices that
 // are added in order first): the results of mixers that run side by side, each normed over the row.
+// PER: values of the row a thread keeps in registers (256 threads x PER cover the width): every slice is read
+// once, and the loads of a slice are asked for together.
+template <int PER>
 __global__ __launch_bounds__(256) void k_normed_sum(const float* __restrict__ a, int a_slices, const float* __restrict__ wa,
                                                     const float* __restrict__ b, int b_slices, const float* __restrict__ wb,
                                                     float* __restrict__ out, int n_tokens, int width, float eps,
                                                     float factor) {
     __shared__ float scratch[16];
     const int t = blockIdx.x;
-    const size_t stride = (size_t)n_tokens * width;
+    const size_t stride = (size_t)n_tokens * width, row = (size_t)t * width;
+    float ya[PER], yb[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) ya[j] = yb[j] = 0.f;
+    for (int s = 0; s < a_slices; ++s)
+#pragma unroll
+        for (int j = 0; j < PER; ++j) ya[j] += a[s * stride + row + min((int)threadIdx.x + j * 256, width - 1)];
+    for (int s = 0; s < b_slices; ++s)
+#pragma unroll
+        for (int j = 0; j < PER; ++j) yb[j] += b[s * stride + row + min((int)threadIdx.x + j * 256, width - 1)];
     float ssa = 0.f, ssb = 0.f;
-    for (int i = threadIdx.x; i < width; i += blockDim.x) {
-        float ya = 0.f, yb = 0.f;
-        for (int s = 0; s < a_slices; ++s) ya += a[s * stride + (size_t)t * width + i];
-        for (int s = 0; s < b_slices; ++s) yb += b[s * stride + (size_t)t * width + i];
-        ssa = fmaf(ya, ya, ssa);
-        ssb = fmaf(yb, yb, ssb);
-    }
+#pragma unroll
+    for (int j = 0; j < PER; ++j)
+        if ((int)threadIdx.x + j * 256 < width) {
+            ssa = fmaf(ya[j], ya[j], ssa);
+            ssb = fmaf(yb[j], yb[j], ssb);
+        }
     const float ra = 1.0f / sqrtf(block_sum(ssa, scratch) / (float)width + eps);
     const float rb = 1.0f / sqrtf(block_sum(ssb, scratch) / (float)width + eps);
-    for (int i = threadIdx.x; i < width; i += blockDim.x) {
-        float ya = 0.f, yb = 0.f;
-        for (int s = 0; s < a_slices; ++s) ya += a[s * stride + (size_t)t * width + i];
-        for (int s = 0; s < b_slices; ++s) yb += b[s * stride + (size_t)t * width + i];
-        out[(size_t)t * width + i] = factor * (ya * ra * wa[i] + yb * rb * wb[i]);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int i = threadIdx.x + j * 256;
+        if (i < width) out[row + i] = factor * (ya[j] * ra * wa[i] + yb[j] * rb * wb[i]);
     }
 }
 
 extern "C" int imparo_normed_sum(const float* a, int a_slices, const float* wa, const float* b, int b_slices,
                                  const float* wb, float* out, int n_tokens, int width, float eps, float factor,
                                  imparo_stream stream) {
-    if (!a || !b || !wa || !wb || !out || a_slices < 1 || b_slices < 1 || n_tokens < 0 || width < 1)
+    if (!a || !b || !wa || !wb || !out || a_slices < 1 || b_slices < 1 || n_tokens < 0 || width < 1 || width > 16384)
         return IMPARO_BAD_ARGUMENT;
     if (n_tokens == 0) return IMPARO_OK;
-    k_normed_sum<<<n_tokens, 256, 0, (hipStream_t)stream>>>(a, a_slices, wa, b, b_slices, wb, out, n_tokens, width, eps,
-                                                            factor);
+    hipStream_t s = (hipStream_t)stream;
+#define NSUM(PER) k_normed_sum<PER><<<n_tokens, 256, 0, s>>>(a, a_slices, wa, b, b_slices, wb, out, n_tokens, width, eps, factor)
+    const int per = (width + 255) / 256;
+    if (per <= 1) NSUM(1);
+    else if (per <= 2) NSUM(2);
+    else if (per <= 4) NSUM(4);
+    else if (per <= 8) NSUM(8);
+    else if (per <= 16) NSUM(16);
+    else if (per <= 32) NSUM(32);
+    else NSUM(64);
+#undef NSUM
     return launch_status();
 }
 
