@@ -181,9 +181,9 @@ int imparo_hgrn2_scan(const float* rows, int ld, int q_off, int f_off, int v_off
 // float32. dim <= 512. chunk_tokens 0: one launch. Otherwise (a multiple of 8; without beta) segments are walked
 // in chunks side by side, in three launches; max_chunks >= ceil(longest segment / chunk_tokens); chunk_state
 // [n_rows * max_chunks, heads, dim, vdim] and chunk_decay [n_rows * max_chunks, heads] float32 are scratch.
-// With beta, chunk_tokens is 0 or imparo_delta_chunk_tokens() (dim at most imparo_delta_chunk_max_dim()): the delta
-// rule in chunks, two launches; chunk_state then holds [n_rows * max_chunks, heads, 2, chunk, chunk] floats and
-// chunk_decay [n_rows * max_chunks, heads, chunk].
+// chunk_tokens = imparo_delta_chunk_tokens() (dim at most imparo_delta_chunk_max_dim()): a segment's chunks in order,
+// small products a chunk, two launches, with or without beta; chunk_state then holds [n_rows * max_chunks, heads, 2,
+// chunk, chunk] floats and chunk_decay [n_rows * max_chunks, heads, 2, chunk]. With beta chunk_tokens is that or 0.
 int imparo_delta_chunk_tokens(void);
 int imparo_delta_chunk_max_dim(void);
 int imparo_decay_scan(const float* q, int q_ld, int q_off, int q_div, const float* k, int k_ld, int k_off, int k_div,

@@ -223,8 +223,10 @@ __global__ void k_decay_carry(float* __restrict__ chunk_state, const float* __re
 #define DVB 32                // value columns a block of the walk
 #define DMAXK 128             // state rows a head at most, in this form
 
+// PLAIN: the recurrence without the delta rule's correction (b = 1, no triangle): M, log g and the steps only.
+template <bool PLAIN>
 __global__ __launch_bounds__(256) void k_delta_chunk_prepare(const DecayScanArgs A) {
-    __shared__ float sk[DC][DMAXK + 1], sq[DC][DMAXK + 1], sL[DC][DC + 1], lg[DC], sb[DC];
+    __shared__ float sk[DC][DMAXK + 1], sq[DC][DMAXK + 1], sL[PLAIN ? 1 : DC][DC + 1], lg[DC], sb[DC];
     const int r = blockIdx.x / A.max_chunks, chunk = blockIdx.x - r * A.max_chunks, h = blockIdx.y;
     const int tid = threadIdx.x, dim = A.dim, heads = A.heads;
     const int n_all = A.seg_len[r];
@@ -239,14 +241,21 @@ __global__ __launch_bounds__(256) void k_delta_chunk_prepare(const DecayScanArgs
         sq[t][k] = t < n ? qv : 0.f;
     }
     if (tid < DC) {
-        float la = 0.f, b = 0.f;
+        float la = 0.f, b = 0.f, dt = 1.f;
         if (tid < n) {
             const size_t row = (size_t)(first + tid);
-            la = -A.rate[h] * ds_softplus(A.step[row * A.step_ld + A.step_off + h] + A.step_bias[h]);
-            b = ds_sigmoid(A.beta[row * A.beta_ld + A.beta_off + h]);
+            if (A.decay_const) {
+                la = logf(fmaxf(A.decay_const[h], 1e-30f));
+            } else {
+                dt = ds_softplus(A.step[row * A.step_ld + A.step_off + h] + A.step_bias[h]);
+                la = -A.rate[h] * dt;
+            }
+            if constexpr (!PLAIN) b = ds_sigmoid(A.beta[row * A.beta_ld + A.beta_off + h]);
         }
         lg[tid] = la;
         sb[tid] = b;
+        // the steps, for a walk that multiplies its values by them
+        A.chunk_decay[((size_t)blockIdx.x * A.heads + h) * (2 * DC) + DC + tid] = dt;
     }
     __syncthreads();
     if (tid == 0) {
@@ -265,16 +274,18 @@ __global__ __launch_bounds__(256) void k_delta_chunk_prepare(const DecayScanArgs
         float kk = 0.f, qk = 0.f;
         if (j <= t) {
             for (int k = 0; k < dim; ++k) {
-                kk = fmaf(sk[t][k], sk[j][k], kk);
+                if constexpr (!PLAIN) kk = fmaf(sk[t][k], sk[j][k], kk);
                 qk = fmaf(sq[t][k], sk[j][k], qk);
             }
             const float w = expf(lg[t] - lg[j]);
             kk *= w * sb[t];
             qk *= w;
         }
-        sL[t][j] = j < t ? kk : 0.f;
+        if constexpr (!PLAIN) sL[t][j] = j < t ? kk : 0.f;
         M_out[i] = qk;
     }
+    if (tid < DC) A.chunk_decay[at * (2 * DC) + tid] = lg[tid];
+    if constexpr (PLAIN) return;
     __syncthreads();
     if (tid < DC) {
         // column tid of (I + L)^-1 by forward substitution, then times b of that column
@@ -289,24 +300,23 @@ __global__ __launch_bounds__(256) void k_delta_chunk_prepare(const DecayScanArgs
         const float b = sb[tid];
 #pragma unroll
         for (int t = 0; t < DC; ++t) T_out[t * DC + tid] = x[t] * b;
-        A.chunk_decay[at * DC + tid] = lg[tid];
     }
 }
 
 // What a block of the walk asks of memory for one chunk, in registers: asked for while the chunk before is worked on.
 #define DPIECES (DC * DMAXK / 256)        // elements of a chunk's K (and Q) a thread brings at most
 struct DeltaFetch {
-    float k[DPIECES], q[DPIECES], t[DC * DC / 256], m[DC * DC / 256], v[DC / 8], l, last;
+    float k[DPIECES], q[DPIECES], t[DC * DC / 256], m[DC * DC / 256], v[DC / 8], dt[DC / 8], l, last;
 };
 
-template <int VB>
+template <int VB, bool PLAIN>
 __global__ __launch_bounds__(256) void k_delta_chunk_scan(const DecayScanArgs A) {
     constexpr int KLD = DMAXK + 4;                       // floats between two tokens' rows: whole 16-byte pieces
     constexpr int NG = 256 / VB;                         // threads a value column: each takes every NG-th token
     constexpr int TPT = DC / NG;                         // tokens of a chunk a thread takes
     constexpr int KPT = DMAXK / NG;                      // state rows of its column a thread takes at most
     __shared__ __attribute__((aligned(16))) float sk[DC][KLD], sq[DC][KLD];
-    __shared__ float sS[DMAXK][VB], sU[DC][VB], sT[DC][DC], sM[DC][DC], sg[DC], sw[DC];
+    __shared__ float sS[DMAXK][VB], sU[DC][VB], sT[PLAIN ? 1 : DC][DC], sM[DC][DC], sg[DC], sw[DC];
     float (*sR)[VB] = reinterpret_cast<float (*)[VB]>(&sq[0][0]);        // R lies where Q lay, once Q has been used
     const int r = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * VB;
     const int tid = threadIdx.x, v = tid % VB, g = tid / VB;
@@ -339,19 +349,21 @@ __global__ __launch_bounds__(256) void k_delta_chunk_scan(const DecayScanArgs A)
         }
 #pragma unroll
         for (int it = 0; it < DC * DC / 256; ++it) {
-            f.t[it] = T_in[tid + 256 * it];
+            if constexpr (!PLAIN) f.t[it] = T_in[tid + 256 * it];
             f.m[it] = T_in[DC * DC + tid + 256 * it];
         }
-        f.l = A.chunk_decay[at * DC + (tid & (DC - 1))];
-        f.last = A.chunk_decay[at * DC + DC - 1];
+        f.l = A.chunk_decay[at * (2 * DC) + (tid & (DC - 1))];
+        f.last = A.chunk_decay[at * (2 * DC) + DC - 1];
 #pragma unroll
         for (int i = 0; i < TPT; ++i) {
             const int t = min(g + NG * i, n - 1);
             f.v[i] = A.v[(size_t)(first + t) * A.v_ld + A.v_off + h * vdim + min(v0 + v, vdim - 1)];
+            f.dt[i] = A.chunk_decay[at * (2 * DC) + DC + t];
         }
     };
     fetch(0);
     const int kpt = (((dim4 + NG - 1) / NG) + 3) & ~3;   // this thread's state rows: kpt from g * kpt on
+    const float skip = (PLAIN && A.skip) ? A.skip[h] : 0.f;
     for (int chunk = 0; chunk < n_chunks; ++chunk) {
         const int first = A.seg_start[r] + chunk * DC, n = min(DC, n_all - chunk * DC);
         __syncthreads();                                 // the chunk before has been used, the state is whole
@@ -367,16 +379,19 @@ __global__ __launch_bounds__(256) void k_delta_chunk_scan(const DecayScanArgs A)
 #pragma unroll
         for (int it = 0; it < DC * DC / 256; ++it) {
             const int i = tid + 256 * it;
-            sT[i / DC][i % DC] = f.t[it];
+            if constexpr (!PLAIN) sT[i / DC][i % DC] = f.t[it];
             sM[i / DC][i % DC] = f.m[it];
         }
         if (tid < DC) {
             sg[tid] = expf(f.l);
             sw[tid] = expf(f.last - f.l);
         }
-        float vt[TPT];
+        float vt[TPT], dts[TPT];
 #pragma unroll
-        for (int i = 0; i < TPT; ++i) vt[i] = (g + NG * i < n && live) ? f.v[i] : 0.f;
+        for (int i = 0; i < TPT; ++i) {
+            vt[i] = (g + NG * i < n && live) ? f.v[i] : 0.f;
+            dts[i] = f.dt[i];
+        }
         __syncthreads();
         fetch(min(chunk + 1, n_chunks - 1));             // on its way while this chunk is worked on (no load under a branch)
         // what the state says of the chunk's keys and queries
@@ -390,7 +405,7 @@ __global__ __launch_bounds__(256) void k_delta_chunk_scan(const DecayScanArgs A)
             for (int i = 0; i < TPT; ++i) {
                 const float4 kk = *reinterpret_cast<const float4*>(&sk[g + NG * i][k]);
                 const float4 qq = *reinterpret_cast<const float4*>(&sq[g + NG * i][k]);
-                p[i] = fmaf(kk.w, s3, fmaf(kk.z, s2, fmaf(kk.y, s1, fmaf(kk.x, s0, p[i]))));
+                if constexpr (!PLAIN) p[i] = fmaf(kk.w, s3, fmaf(kk.z, s2, fmaf(kk.y, s1, fmaf(kk.x, s0, p[i]))));
                 s[i] = fmaf(qq.w, s3, fmaf(qq.z, s2, fmaf(qq.y, s1, fmaf(qq.x, s0, s[i]))));
             }
         }
@@ -398,25 +413,30 @@ __global__ __launch_bounds__(256) void k_delta_chunk_scan(const DecayScanArgs A)
 #pragma unroll
         for (int i = 0; i < TPT; ++i) {
             const int t = g + NG * i;
-            sR[t][v] = vt[i] - sg[t] * p[i];
+            if constexpr (PLAIN)
+                sU[t][v] = A.v_times_step ? vt[i] * dts[i] : vt[i];     // no correction: what is written is the value itself
+            else
+                sR[t][v] = vt[i] - sg[t] * p[i];
             s[i] *= sg[t];
         }
         for (int i = tid; i < DC * dim4; i += 256) sk[i / dim4][i % dim4] *= sw[i / dim4];
         __syncthreads();
         // (T and M are zero above their diagonals: the sums run over the whole chunk, so that the reads of
         // several steps can be under way at once; a product with zero adds nothing)
-        float u[TPT];
+        if constexpr (!PLAIN) {
+            float u[TPT];
 #pragma unroll
-        for (int i = 0; i < TPT; ++i) u[i] = 0.f;
+            for (int i = 0; i < TPT; ++i) u[i] = 0.f;
 #pragma unroll 8
-        for (int j = 0; j < DC; ++j) {
-            const float rv = sR[j][v];
+            for (int j = 0; j < DC; ++j) {
+                const float rv = sR[j][v];
 #pragma unroll
-            for (int i = 0; i < TPT; ++i) u[i] = fmaf(sT[g + NG * i][j], rv, u[i]);
+                for (int i = 0; i < TPT; ++i) u[i] = fmaf(sT[g + NG * i][j], rv, u[i]);
+            }
+#pragma unroll
+            for (int i = 0; i < TPT; ++i) sU[g + NG * i][v] = u[i];
+            __syncthreads();
         }
-#pragma unroll
-        for (int i = 0; i < TPT; ++i) sU[g + NG * i][v] = u[i];
-        __syncthreads();
 #pragma unroll 8
         for (int j = 0; j < DC; ++j) {
             const float uv = sU[j][v];
@@ -426,7 +446,8 @@ __global__ __launch_bounds__(256) void k_delta_chunk_scan(const DecayScanArgs A)
 #pragma unroll
         for (int i = 0; i < TPT; ++i) {
             const int t = g + NG * i;
-            if (t < n && live) A.out[(size_t)(first + t) * heads * vdim + (size_t)h * vdim + v0 + v] = s[i];
+            if (t < n && live)
+                A.out[(size_t)(first + t) * heads * vdim + (size_t)h * vdim + v0 + v] = PLAIN ? fmaf(skip, vt[i], s[i]) : s[i];
         }
         // the state behind the chunk: this thread's rows of its column
         const float g_last = sg[DC - 1];
@@ -474,6 +495,7 @@ extern "C" int imparo_decay_scan(const float* q, int q_ld, int q_off, int q_div,
     if (chunk_tokens < 0 || chunk_tokens % DS_TOKENS) return IMPARO_BAD_ARGUMENT;
     if (chunk_tokens && (max_chunks < 1 || !chunk_state || !chunk_decay)) return IMPARO_BAD_ARGUMENT;
     if (chunk_tokens && beta && (chunk_tokens != DC || dim > DMAXK || decay_const)) return IMPARO_BAD_ARGUMENT;
+    if (chunk_tokens == DC && dim > DMAXK) return IMPARO_BAD_ARGUMENT;
     if (n_rows < 0 || heads < 1 || dim < 1 || dim > DS_MAX_DIM || vdim < 1) return IMPARO_BAD_ARGUMENT;
     if (q_div < 1 || k_div < 1 || heads % q_div || heads % k_div) return IMPARO_BAD_ARGUMENT;
     if (q_off < 0 || k_off < 0 || v_off < 0 || q_ld < q_off + heads / q_div * dim || k_ld < k_off + heads / k_div * dim ||
@@ -497,19 +519,23 @@ extern "C" int imparo_decay_scan(const float* q, int q_ld, int q_off, int q_div,
                              step, step_ld, step_off, step_bias, rate, v_times_step, beta, beta_ld, beta_off, skip,
                              state, seg_start, seg_len, slot, out, heads, dim, vdim, kpt,
                              chunk_tokens, max_chunks, chunk_state, chunk_decay};
-    if (beta && chunk_tokens) {
-        // the delta rule in chunks: chunk_state holds T and M of every chunk, chunk_decay the logarithms of its decays
-        if (v_times_step || skip) return IMPARO_BAD_ARGUMENT;
-        k_delta_chunk_prepare<<<dim3(n_rows * max_chunks, heads), 256, 0, s>>>(args);
+    if (chunk_tokens == DC && dim <= DMAXK) {
+        // the chunks of a segment in order, small products a chunk: chunk_state holds T and M of every chunk,
+        // chunk_decay the logarithms of its decays and its steps
+        if (beta && (v_times_step || skip)) return IMPARO_BAD_ARGUMENT;
+        const dim3 pgrid(n_rows * max_chunks, heads);
+        if (beta) k_delta_chunk_prepare<false><<<pgrid, 256, 0, s>>>(args);
+        else k_delta_chunk_prepare<true><<<pgrid, 256, 0, s>>>(args);
         // few blocks (a segment, few heads): narrower runs of columns make more of them
         // (a column's arithmetic is the same whatever the width of its run: the same bits)
         const long long rh = (long long)n_rows * heads;
-        if (rh * ((vdim + DVB - 1) / DVB) >= 256 || vdim <= 8)
-            k_delta_chunk_scan<DVB><<<dim3(n_rows, heads, (vdim + DVB - 1) / DVB), 256, 0, s>>>(args);
-        else if (rh * ((vdim + 15) / 16) >= 256 || vdim <= 8)
-            k_delta_chunk_scan<16><<<dim3(n_rows, heads, (vdim + 15) / 16), 256, 0, s>>>(args);
-        else
-            k_delta_chunk_scan<8><<<dim3(n_rows, heads, (vdim + 7) / 8), 256, 0, s>>>(args);
+#define DCS(VB)                                                                                                      \
+    if (beta) k_delta_chunk_scan<VB, false><<<dim3(n_rows, heads, (vdim + VB - 1) / VB), 256, 0, s>>>(args);        \
+    else k_delta_chunk_scan<VB, true><<<dim3(n_rows, heads, (vdim + VB - 1) / VB), 256, 0, s>>>(args)
+        if (rh * ((vdim + DVB - 1) / DVB) >= 512 || vdim <= 8) { DCS(DVB); }
+        else if (rh * ((vdim + 15) / 16) >= 512) { DCS(16); }
+        else { DCS(8); }
+#undef DCS
         return launch_status();
     }
 #define DS_PASS(KS, MODE, DELTA)                                                                                     \

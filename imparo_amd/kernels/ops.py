@@ -1138,25 +1138,29 @@ DECAY_SCAN_MAX_DIM = 512          # state rows a head
 DECAY_SCAN_CHUNK = 64             # tokens a chunk when a long segment's chunks run side by side
 
 
-def decay_scan_chunks(max_seg_len: int, delta: bool = False, dim: int = 0):
-    """(chunk_tokens, max_chunks) for `decay_scan`: (0, 1) for one launch, which short segments take; else chunks
-    of DECAY_SCAN_CHUNK tokens (the delta rule: of its own chunk size, for heads of up to its largest dim), as
-    many as the longest segment makes."""
-    if delta:
-        chunk = int(library().imparo_delta_chunk_tokens())
-        if max_seg_len < 2 * chunk or dim > int(library().imparo_delta_chunk_max_dim()):
+def decay_scan_chunks(max_seg_len: int, delta: bool = False, dim: int = 0, blocks: int = 0):
+    """(chunk_tokens, max_chunks) for `decay_scan`: (0, 1) for one launch, which short segments take. Heads of up
+    to the chunk form's largest dim: a segment's chunks in order, small products a chunk (the form the delta rule
+    needs, and the faster one for a plain decay too where it fills the chip). Wider heads with a plain decay: chunks
+    of DECAY_SCAN_CHUNK tokens side by side; wider heads of the delta rule: token by token."""
+    chunk = int(library().imparo_delta_chunk_tokens())
+    # `blocks`: segments x heads x runs of 8 value columns, the most blocks the chunks-in-order form can make. Where
+    # that does not fill the chip, a plain decay's long segments run their chunks side by side instead.
+    side_by_side = not delta and 0 < blocks < 256 and max_seg_len >= 4 * DECAY_SCAN_CHUNK
+    if dim <= int(library().imparo_delta_chunk_max_dim()) and not side_by_side:
+        if max_seg_len < 2 * chunk:
             return 0, 1
         return chunk, -(-int(max_seg_len) // chunk)
-    if max_seg_len < 4 * DECAY_SCAN_CHUNK:
+    if delta or max_seg_len < 4 * DECAY_SCAN_CHUNK:
         return 0, 1
     return DECAY_SCAN_CHUNK, -(-int(max_seg_len) // DECAY_SCAN_CHUNK)
 
 
-def decay_scan_scratch(n_rows: int, max_chunks: int, heads: int, dim: int, vdim: int, delta: bool = False):
-    """Floats of (chunk_state, chunk_decay) that `decay_scan` needs when it walks in chunks."""
-    if delta:
-        chunk = int(library().imparo_delta_chunk_tokens())
-        return n_rows * max_chunks * heads * 2 * chunk * chunk, n_rows * max_chunks * heads * chunk
+def decay_scan_scratch(n_rows: int, max_chunks: int, heads: int, dim: int, vdim: int, chunk_tokens: int):
+    """Floats of (chunk_state, chunk_decay) that `decay_scan` needs when it walks in chunks of `chunk_tokens`."""
+    chunk = int(library().imparo_delta_chunk_tokens())
+    if chunk_tokens == chunk:
+        return n_rows * max_chunks * heads * 2 * chunk * chunk, n_rows * max_chunks * heads * 2 * chunk
     return n_rows * max_chunks * heads * dim * vdim, n_rows * max_chunks * heads
 
 
@@ -1183,7 +1187,7 @@ def decay_scan(q: torch.Tensor, q_off: int, q_div: int, k: torch.Tensor, k_off: 
     if (decay_const is None) == (step is None):
         raise KernelArgumentError("decay_scan: the decay is a constant a head or comes from projected steps")
     if chunk_tokens:
-        need_s, need_d = decay_scan_scratch(n_rows, max_chunks, heads, dim, vdim, beta is not None)
+        need_s, need_d = decay_scan_scratch(n_rows, max_chunks, heads, dim, vdim, chunk_tokens)
         if chunk_state is None or chunk_decay is None or chunk_state.numel() < need_s or chunk_decay.numel() < need_d:
             raise KernelArgumentError("decay_scan: the scratch for the chunks' states is too small")
     _check(library().imparo_decay_scan(

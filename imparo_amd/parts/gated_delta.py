@@ -120,7 +120,7 @@ class GatedDelta:
         chunk_tokens, max_chunks = ops.decay_scan_chunks(ctx.max_seg_len, delta=True, dim=dk)
         chunk_state = chunk_decay = None
         if chunk_tokens:
-            n_state, n_decay = ops.decay_scan_scratch(ctx.n_rows, max_chunks, H, dk, dv, delta=True)
+            n_state, n_decay = ops.decay_scan_scratch(ctx.n_rows, max_chunks, H, dk, dv, chunk_tokens)
             chunk_state = ctx.workspace.get("scan_chunk_state", (n_state,), torch.float32)
             chunk_decay = ctx.workspace.get("scan_chunk_decay", (n_decay,), torch.float32)
         ops.decay_scan(qkv, 0, H // Hk, qkv, Hk * dk, H // Hk, qkv, 2 * Hk * dk, state["state"], ctx.seg_start,

@@ -113,10 +113,10 @@ class Mamba2:
         ops.causal_conv(rows, C, self.conv_weight, self.conv_bias, state.get("conv"), ctx.row_of_token, ctx.seg_start,
                         ctx.seg_len, ctx.slot, xbc, silu=True, single_tokens=ctx.max_seg_len == 1, u_off=inner)
         y = ctx.workspace.get("ssd_y", (T, inner), torch.float32)
-        chunk_tokens, max_chunks = ops.decay_scan_chunks(ctx.max_seg_len)
+        chunk_tokens, max_chunks = ops.decay_scan_chunks(ctx.max_seg_len, dim=N, blocks=ctx.n_rows * H * -(-P // 8))
         chunk_state = chunk_decay = None
         if chunk_tokens:
-            n_state, n_decay = ops.decay_scan_scratch(ctx.n_rows, max_chunks, H, N, P)
+            n_state, n_decay = ops.decay_scan_scratch(ctx.n_rows, max_chunks, H, N, P, chunk_tokens)
             chunk_state = ctx.workspace.get("scan_chunk_state", (n_state,), torch.float32)
             chunk_decay = ctx.workspace.get("scan_chunk_decay", (n_decay,), torch.float32)
         ops.decay_scan(xbc, inner + G * N, H // G, xbc, inner, H // G, xbc, 0, state["state"], ctx.seg_start, ctx.seg_len,

@@ -92,10 +92,10 @@ class Retention:
                          interleaved=bool(getattr(self.position, "interleaved", False)), positions=ctx.positions,
                          n_first=H, scale_first=1.0, scale_rest=float(d) ** -0.5)
         o = ctx.workspace.get("retention_o", (T, H * dv), torch.float32)
-        chunk_tokens, max_chunks = ops.decay_scan_chunks(ctx.max_seg_len)
+        chunk_tokens, max_chunks = ops.decay_scan_chunks(ctx.max_seg_len, dim=d, blocks=ctx.n_rows * H * -(-dv // 8))
         chunk_state = chunk_decay = None
         if chunk_tokens:
-            n_state, n_decay = ops.decay_scan_scratch(ctx.n_rows, max_chunks, H, d, dv)
+            n_state, n_decay = ops.decay_scan_scratch(ctx.n_rows, max_chunks, H, d, dv, chunk_tokens)
             chunk_state = ctx.workspace.get("scan_chunk_state", (n_state,), torch.float32)
             chunk_decay = ctx.workspace.get("scan_chunk_decay", (n_decay,), torch.float32)
         ops.decay_scan(rows, 0, 1, rows, H * d, 1, rows, 2 * H * d, ctx.fixed_arrays(site)["state"], ctx.seg_start,

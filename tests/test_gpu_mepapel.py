@@ -177,7 +177,7 @@ def test_recurrence_kernel_continues_over_segments_in_used_slots(H, share, d, dv
         chunk_tokens, max_chunks = ops.decay_scan_chunks(max(seg), delta=kind == "delta", dim=d)
         cs = cd = None
         if chunk_tokens:
-            n_state, n_decay = ops.decay_scan_scratch(len(rows), max_chunks, H, d, dv, delta=kind == "delta")
+            n_state, n_decay = ops.decay_scan_scratch(len(rows), max_chunks, H, d, dv, chunk_tokens)
             cs, cd = torch.empty(n_state, device=DEV), torch.empty(n_decay, device=DEV)
         kw = dict(decay_const=dev(const)) if kind == "constant" else dict(
             step=rows_t, step_off=2 * Hs * d + H * dv, step_bias=dev(bias), rate=dev(rate))
