@@ -10,7 +10,7 @@ are one number a head. Per head, with a state S [dim, vdim]:
 
     S <- g S;   u = b (v - S^T k);   S <- S + k u^T;   o = S^T q
 
-(the read-out sees the token's own write). Each head's o is divided by its
+(in that order: a token's result already holds what the token wrote). Each head's o is divided by its
 root mean square, multiplied by a weight that all heads share and by
 silu(Wg h); the heads side by side go through the output projection. A
 request's state is S, float32, and the convs' last taps - 1 inputs. Gates,

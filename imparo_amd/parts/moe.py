@@ -18,7 +18,8 @@ weight; "input": the expert reads its input times its weight and the results
 are added as they are), `group_count` and `group_keep` (the router outputs form
 group_count equal groups of neighbours; a group's score is the sum of its two
 largest score + correction, and only outputs of the group_keep best groups can
-be chosen: the others' choice scores count as minus infinity), `normalize` (the
+be chosen: an output of another group never is, however low the scores
+inside the kept groups lie), `normalize` (the
 chosen scores are divided by their sum + 1e-20), `route_scale` (a factor on the
 weights), `shared` (the PartSpec of a feed-forward that every token uses; its
 result is added, multiplied by sigmoid(Wsg n), one number a token, with Wsg the

@@ -301,7 +301,8 @@ def test_small_kernels_of_the_feed_forwards_and_the_pair():
                                                (130, 2, 1, 5), (4, 2, 2, 4)])
 def test_route_kernel_with_groups(X, groups, keep, top):
     """Sigmoid scores, the choice by score + correction among the outputs of the best groups only (a group scores
-    the sum of its two largest choice scores; negative choice scores must not beat minus infinity), weights the
+    the sum of its two largest choice scores; with mostly negative choice scores, so that a group shut out by
+    a zero instead of minus infinity would show), weights the
     chosen scores over their sum times a factor; logits read from rows that hold one more column."""
     from imparo_amd.kernels import ops
     g = torch.Generator().manual_seed(X + top)
