@@ -297,6 +297,43 @@ def test_small_kernels_of_the_feed_forwards_and_the_pair():
     assert torch.equal(out.cpu(), stream.cpu().to(torch.bfloat16))
 
 
+@pytest.mark.parametrize("taps,silu,bias", [(4, True, True), (3, False, False), (2, True, False), (1, False, True)])
+def test_conv_over_columns_inside_a_wider_row(taps, silu, bias):
+    """The short conv over channels that start at a column offset of a fused projection's rows, continued over
+    segments of 1 to 40 tokens (shorter than the history too) in used slots, with and without activation and bias."""
+    from imparo_amd.kernels import ops
+    g = torch.Generator().manual_seed(taps)
+    C, off, ld, lens, slots = 20, 7, 33, [46, 3, 9], [2, 0, 3]
+    cuts = [[1, 2, 40, 3], [3], [1, 1, 7]]
+    w, b = torch.randn(C, taps, generator=g), torch.randn(C, generator=g)
+    rows = [torch.randn(n, ld, generator=g) for n in lens]
+    want = []
+    for x in rows:
+        y = plain.causal_conv(x[:, off:off + C].double(), w.double(), b.double() if bias else None)
+        want.append(plain.silu(y) if silu else y)
+    state = torch.randn(4, max(taps - 1, 1), C, generator=g)
+    st = dev(state)
+    for r in slots:
+        st[r].zero_()
+    fed, got = [0, 0, 0], [[] for _ in lens]
+    while any(fed[r] < lens[r] for r in range(3)):
+        live = [r for r in range(3) if fed[r] < lens[r]]
+        seg = [cuts[r].pop(0) for r in live]
+        u = dev(torch.cat([rows[r][fed[r]:fed[r] + n] for r, n in zip(live, seg)]))
+        starts = np.cumsum([0] + seg[:-1])
+        row_of = np.concatenate([[i] * n for i, n in enumerate(seg)])
+        out = torch.empty(u.shape[0], C, device=DEV)
+        ops.causal_conv(u, C, dev(w), dev(b) if bias else None, st if taps > 1 else None, i32(row_of), i32(starts), i32(seg),
+                        i32([slots[r] for r in live]), out, silu=silu, single_tokens=max(seg) == 1, u_off=off)
+        at = 0
+        for r, n in zip(live, seg):
+            got[r].append(out[at:at + n].cpu())
+            at += n
+            fed[r] += n
+    for r in range(3):
+        near(torch.cat(got[r]), want[r], 3e-6, f"request {r}")
+
+
 @pytest.mark.parametrize("X,groups,keep,top", [(6, 3, 2, 2), (8, 4, 1, 2), (16, 4, 2, 4), (12, 1, 1, 3), (8, 8, 3, 3), (64, 8, 2, 8),
                                                (130, 2, 1, 5), (4, 2, 2, 4)])
 def test_route_kernel_with_groups(X, groups, keep, top):
