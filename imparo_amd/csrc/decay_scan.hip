@@ -619,46 +619,72 @@ extern "C" int imparo_head_prepare(float* rows, int ld, int off, int n_tokens, i
 // ---------------------------------------------------------------- the heads behind the walk
 // out[t, c] for a row of `width` values in `groups` equal parts: with y = x[t, c] and g = silu(gate[t, c]),
 //   gate_first: (y g) / rms_part(y g) * w[c];   otherwise: y / rms_part(y) * w[c] * g     (w null: 1).
-// A wave takes a part (WHOLE_BLOCK: a block does, for long parts).
-template <typename TOut, bool WHOLE_BLOCK>
+// A wave takes a part; for long parts a block does, with the part in registers (PER values a thread, every load
+// asked for before any is used, the gate's activation taken once).
+template <typename TOut>
 __global__ __launch_bounds__(256) void k_gated_group_norm(const float* __restrict__ x, const float* __restrict__ gate,
                                                           int gate_ld, int gate_off, const float* __restrict__ w,
                                                           TOut* __restrict__ out, int n_tokens, int width, int groups,
                                                           float eps, int gate_first) {
-    __shared__ float scratch[16];
     const int part = width / groups;
-    long long id;
-    int first, stride;
-    if (WHOLE_BLOCK) {
-        id = blockIdx.x;
-        first = threadIdx.x;
-        stride = blockDim.x;
-    } else {
-        id = (long long)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
-        first = threadIdx.x & (WAVE - 1);
-        stride = WAVE;
-        if (id >= (long long)n_tokens * groups) return;
-    }
+    const long long id = (long long)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    const int first = threadIdx.x & (WAVE - 1);
+    if (id >= (long long)n_tokens * groups) return;
     const int t = (int)(id / groups), g = (int)(id - (long long)t * groups);
     const float* xr = x + (size_t)t * width + (size_t)g * part;
     const float* gr = gate ? gate + (size_t)t * gate_ld + gate_off + (size_t)g * part : nullptr;
     float ss = 0.f;
 #pragma unroll 4
-    for (int i = first; i < part; i += stride) {
+    for (int i = first; i < part; i += WAVE) {
         float y = xr[i];
         if (gate_first && gr) y *= ds_silu(gr[i]);
         ss = fmaf(y, y, ss);
     }
-    ss = WHOLE_BLOCK ? block_sum(ss, scratch) : wave_sum(ss);
+    ss = wave_sum(ss);
     const float rs = 1.0f / sqrtf(ss / (float)part + eps);
 #pragma unroll 4
-    for (int i = first; i < part; i += stride) {
+    for (int i = first; i < part; i += WAVE) {
         float y = xr[i];
         const float gv = gr ? ds_silu(gr[i]) : 1.f;
         if (gate_first) y *= gv;
         y = y * rs * (w ? w[(size_t)g * part + i] : 1.f);
         if (!gate_first) y *= gv;
         store_f32<TOut>(out, (size_t)t * width + (size_t)g * part + i, y);
+    }
+}
+
+template <typename TOut, int PER>
+__global__ __launch_bounds__(256) void k_gated_group_norm_block(const float* __restrict__ x, const float* __restrict__ gate,
+                                                                int gate_ld, int gate_off, const float* __restrict__ w,
+                                                                TOut* __restrict__ out, int width, int groups, float eps,
+                                                                int gate_first) {
+    __shared__ float scratch[16];
+    const int part = width / groups;
+    const int t = blockIdx.x / groups, g = blockIdx.x - t * groups;
+    const float* xr = x + (size_t)t * width + (size_t)g * part;
+    const float* gr = gate ? gate + (size_t)t * gate_ld + gate_off + (size_t)g * part : nullptr;
+    float y[PER], gv[PER], wv[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int i = min((int)threadIdx.x + j * 256, part - 1);
+        y[j] = xr[i];
+        gv[j] = gr ? gr[i] : 0.f;
+        wv[j] = w ? w[(size_t)g * part + i] : 1.f;
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        gv[j] = gr ? ds_silu(gv[j]) : 1.f;
+        if (gate_first) y[j] *= gv[j];
+        if ((int)threadIdx.x + j * 256 < part) ss = fmaf(y[j], y[j], ss);
+    }
+    const float rs = 1.0f / sqrtf(block_sum(ss, scratch) / (float)part + eps);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int i = threadIdx.x + j * 256;
+        float v = y[j] * rs * wv[j];
+        if (!gate_first) v *= gv[j];
+        if (i < part) store_f32<TOut>(out, (size_t)t * width + (size_t)g * part + i, v);
     }
 }
 
@@ -672,16 +698,29 @@ extern "C" int imparo_gated_group_norm(const float* x, const float* gate, int ga
     hipStream_t s = (hipStream_t)stream;
     const long long parts = (long long)n_tokens * groups;
     if (parts > 0x7fffffffLL) return IMPARO_BAD_ARGUMENT;
-    const bool whole = width / groups > 512;
-#define GGN(T, WHOLE, BLOCKS)                                                                                        \
-    k_gated_group_norm<T, WHOLE><<<(unsigned)(BLOCKS), 256, 0, s>>>(x, gate, gate_ld, gate_off, w, (T*)out, n_tokens, \
-                                                                    width, groups, eps, gate_first)
-    if (out_dtype == IMPARO_BF16) {
-        if (whole) GGN(bf16_t, true, parts); else GGN(bf16_t, false, (parts + 3) / 4);
-    } else {
-        if (whole) GGN(float, true, parts); else GGN(float, false, (parts + 3) / 4);
+    const int part = width / groups;
+    if (part > 512 && part <= 256 * 64) {
+#define GGN_BLOCK(T, PER)                                                                                            \
+    k_gated_group_norm_block<T, PER><<<(unsigned)parts, 256, 0, s>>>(x, gate, gate_ld, gate_off, w, (T*)out, width, \
+                                                                     groups, eps, gate_first)
+#define GGN_PER(T)                                                                                                   \
+    if (part <= 256 * 4) GGN_BLOCK(T, 4);                                                                            \
+    else if (part <= 256 * 8) GGN_BLOCK(T, 8);                                                                       \
+    else if (part <= 256 * 16) GGN_BLOCK(T, 16);                                                                     \
+    else if (part <= 256 * 32) GGN_BLOCK(T, 32);                                                                     \
+    else GGN_BLOCK(T, 64)
+        if (out_dtype == IMPARO_BF16) { GGN_PER(bf16_t); } else { GGN_PER(float); }
+#undef GGN_PER
+#undef GGN_BLOCK
+        return launch_status();
     }
-#undef GGN
+    const unsigned blocks = (unsigned)((parts + 3) / 4);
+    if (out_dtype == IMPARO_BF16)
+        k_gated_group_norm<bf16_t><<<blocks, 256, 0, s>>>(x, gate, gate_ld, gate_off, w, (bf16_t*)out, n_tokens, width,
+                                                          groups, eps, gate_first);
+    else
+        k_gated_group_norm<float><<<blocks, 256, 0, s>>>(x, gate, gate_ld, gate_off, w, (float*)out, n_tokens, width,
+                                                         groups, eps, gate_first);
     return launch_status();
 }
 
