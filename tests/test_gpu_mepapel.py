@@ -297,6 +297,36 @@ def test_small_kernels_of_the_feed_forwards_and_the_pair():
     assert torch.equal(out.cpu(), stream.cpu().to(torch.bfloat16))
 
 
+def test_a_place_for_a_norm_without_one():
+    """The norm kind `none`: the stream itself in the reader's dtype; a pending delta is added first, through the
+    norm it carries (in slices too) or as it is; a float32 reader with nothing pending gets the stream, no copy."""
+    from imparo_amd.config.plan import PartSpec
+    from imparo_amd.parts import part_class
+    from imparo_amd.parts.base import Residual
+    g = torch.Generator().manual_seed(9)
+    T, E = 6, 40
+    part = part_class("norm", "none")(PartSpec("none", "", dict(width=E)), {}, torch.device(DEV), torch.bfloat16)
+    ctx = hand_context([(0, T)], 16, 2, torch.bfloat16, torch.device(DEV))
+    x, d, wp = torch.randn(T, E, generator=g), torch.randn(3, T, E, generator=g), torch.rand(E, generator=g) + 0.5
+    res = Residual(dev(x))
+    assert part.forward(ctx, res, torch.float32) is res.x
+    assert torch.equal(part.forward(ctx, res, torch.bfloat16).cpu(), x.to(torch.bfloat16))
+    res = Residual(dev(x), pending=dev(d))                      # slices without a norm: added in order
+    out = part.forward(ctx, res, torch.bfloat16)
+    want = x.double() + d.double().sum(0)
+    near(res.x.cpu(), want, 3e-6)
+    assert res.pending is None and torch.equal(out.cpu(), res.x.cpu().to(torch.bfloat16))
+    res = Residual(dev(x), pending=dev(d), post=(dev(wp), 1e-5))
+    out = part.forward(ctx, res, torch.float32, name="other")
+    want = x.double() + plain.unit_rms(d.double().sum(0), 1e-5) * wp
+    near(out.cpu(), want, 3e-6)
+    assert res.pending is None and res.post is None and torch.equal(out.cpu(), res.x.cpu())
+    res = Residual(dev(x), pending=dev(d), post=(dev(wp), 1e-5))
+    rows = part.forward_rows(ctx, res, i32([4, 1]), torch.float32)
+    near(rows.cpu(), want[[4, 1]], 3e-6)
+    assert torch.equal(res.x.cpu(), x)                           # chosen rows only: the stream stays
+
+
 @pytest.mark.parametrize("taps,silu,bias", [(4, True, True), (3, False, False), (2, True, False), (1, False, True)])
 def test_conv_over_columns_inside_a_wider_row(taps, silu, bias):
     """The short conv over channels that start at a column offset of a fused projection's rows, continued over
